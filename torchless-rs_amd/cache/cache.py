@@ -53,6 +53,13 @@ class KVRequest:
     def value_dim(self) -> int:
         return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
+    def covering(self, window: Optional[int]) -> "KVRequest":
+        """The request that also serves a reader who looks back `window` positions (None: to the
+        first): the wider of the two windows, none if either has none."""
+        if self.window is None or (window is not None and window <= self.window):
+            return self
+        return KVRequest(self.n_kv_heads, self.head_dim, window, self.v_head_dim)
+
 
 @dataclass(frozen=True)
 class StateRequest:

@@ -70,8 +70,11 @@ def get_architecture(name: str) -> ArchitectureEntry:
 
 def architecture_name(d: Dict[str, Any]) -> str:
     archs = d.get("architectures")
+    if archs is None and isinstance(d.get("architecture"), str):
+        return d["architecture"]             # some files name their one design in a plain string
     if not isinstance(archs, (list, tuple)) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json: 'architectures' must be a non-empty list of names")
+        raise ConfigError("config.json: 'architectures' must be a non-empty list of names "
+                          "(or 'architecture' one name)")
     return archs[0]
 
 

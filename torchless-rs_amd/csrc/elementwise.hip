@@ -458,6 +458,122 @@ __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chu
   *reinterpret_cast<bf16x8*>(out + n * I + group * 32 + part * 8) = o;
 }
 
+// ---- layer norm with a weight and no bias: y = (x - mean) / sqrt(var + eps) * w -------------
+// var is the mean of the squared deviations from the mean (two passes over the row, both in
+// float).  The row may get a bias first (z + b, the bias of the product that made z).
+// `x` null: y is written to `out`.  `x` given: the norm is ADDED to the stream, x += y, and
+// `out` (may be null) receives the new x in the compute type, for the product that reads
+// the stream next.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+layernorm_kernel(const float* __restrict__ z, const float* __restrict__ bias, const float* __restrict__ w,
+                 float eps, float* __restrict__ x, TO* __restrict__ out, int H) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x;
+  const float* zr = z + (size_t)n * H;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) s += zr[i] + (bias ? bias[i] : 0.f);
+  const float mean = block_sum<256>(s, sh) / (float)H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float d = zr[i] + (bias ? bias[i] : 0.f) - mean;
+    ss += d * d;
+  }
+  const float sd = sqrtf(block_sum<256>(ss, sh) / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float y = ((zr[i] + (bias ? bias[i] : 0.f) - mean) / sd) * w[i];
+    if (x) {
+      const float xn = x[(size_t)n * H + i] + y;
+      x[(size_t)n * H + i] = xn;
+      if (out) out[(size_t)n * H + i] = from_f32<TO>(xn);
+    } else {
+      out[(size_t)n * H + i] = from_f32<TO>(y);
+    }
+  }
+}
+
+// The same with the row held in registers: one read of z.  H % 4 == 0, H <= 1024 * IT.
+template <typename TO, int IT>
+__global__ void __launch_bounds__(256)
+layernorm_reg_kernel(const float* __restrict__ z, const float* __restrict__ bias, const float* __restrict__ w,
+                     float eps, float* __restrict__ x, TO* __restrict__ out, int H) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x;
+  const float4* zr = reinterpret_cast<const float4*>(z + (size_t)n * H);
+  const float4* br = reinterpret_cast<const float4*>(bias);
+  const float4* wr = reinterpret_cast<const float4*>(w);
+  const int nv = H / 4;
+  float4 v[IT];
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      v[i] = zr[c];
+      if (bias) {
+        const float4 b = br[c];
+        v[i].x += b.x; v[i].y += b.y; v[i].z += b.z; v[i].w += b.w;
+      }
+      s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+  }
+  const float mean = block_sum<256>(s, sh) / (float)H;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      v[i].x -= mean; v[i].y -= mean; v[i].z -= mean; v[i].w -= mean;
+      ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+  }
+  const float sd = sqrtf(block_sum<256>(ss, sh) / (float)H + eps);
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      const float4 g = wr[c];
+      float4 y;
+      y.x = (v[i].x / sd) * g.x; y.y = (v[i].y / sd) * g.y; y.z = (v[i].z / sd) * g.z; y.w = (v[i].w / sd) * g.w;
+      if (x) {
+        float4* xr = reinterpret_cast<float4*>(x + (size_t)n * H);
+        float4 a = xr[c];
+        a.x += y.x; a.y += y.y; a.z += y.z; a.w += y.w;
+        xr[c] = a;
+        y = a;
+        if (!out) continue;
+      }
+      TO* o = out + (size_t)n * H + 4 * c;
+      o[0] = from_f32<TO>(y.x); o[1] = from_f32<TO>(y.y); o[2] = from_f32<TO>(y.z); o[3] = from_f32<TO>(y.w);
+    }
+  }
+}
+
+// out = x in bfloat16, for a product that reads the stream itself
+__global__ void cast_rows_kernel(const float* __restrict__ x, size_t total, bf16* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) out[i] = (bf16)x[i];
+}
+
+// ---- the function of a gated feed-forward's gate ---------------------------------
+// 0: silu(g) = g / (1 + exp(-g)); 1: the tanh form of gelu,
+// 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+constexpr int ACT_SILU = 0;
+constexpr int ACT_GELU_TANH = 1;
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.0f + expf(-g));
+}
+
+// h = act(gate) * up from gu[n, 2I] = [gate | up]
+template <typename TO>
+__global__ void act_mul_kernel(const float* __restrict__ gu, int I, int act, TO* __restrict__ out) {
+  const int n = blockIdx.x;
+  const float* row = gu + (size_t)n * 2 * I;
+  for (int i = threadIdx.x; i < I; i += blockDim.x)
+    out[(size_t)n * I + i] = from_f32<TO>(gate_act(row[i], act) * row[I + i]);
+}
+
 // tokens[j] = src[idx[j]]: the ids that the sampler left on the device become the next step's
 // input without a trip to the host.  An id outside the vocabulary becomes 0 (no row of the
 // embedding lies there).
@@ -735,6 +851,54 @@ int tl_silu_mul_pairs(const void* gu, int n, int I, void* out, hipStream_t st) {
   TL_REQUIRE((chunks + 255) / 256 < 2147483647LL, "silu_mul_pairs: too many elements");
   silu_mul_pairs_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const bf16*)gu, chunks, I, (bf16*)out);
   TL_LAUNCH_CHECK("silu_mul_pairs");
+  return 0;
+}
+
+// x null: out = layernorm(z + bias); else x += layernorm(z + bias) and out (may be null) = x
+int tl_layernorm(const float* z, const float* bias, const float* w, float eps, float* x, void* out, int out_dt,
+                 int n, int H, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0, "layernorm: bad sizes n=%d H=%d", n, H);
+  TL_REQUIRE(x != nullptr || out != nullptr, "layernorm: nowhere to write");
+  TL_REQUIRE(out == nullptr || out_dt == DT_F32 || out_dt == DT_BF16, "layernorm: unknown dtype code %d", out_dt);
+  if (n == 0) return 0;
+  const bool al = (uintptr_t)z % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)bias % 16 == 0 && (uintptr_t)x % 16 == 0;
+  const bool vec = H % 4 == 0 && H <= 8192 && al;
+  const bool f32 = out == nullptr || out_dt == DT_F32;
+#define TL_LN(IT)                                                                                        \
+  do {                                                                                                   \
+    if (f32) layernorm_reg_kernel<float, IT><<<n, 256, 0, st>>>(z, bias, w, eps, x, (float*)out, H);     \
+    else layernorm_reg_kernel<bf16, IT><<<n, 256, 0, st>>>(z, bias, w, eps, x, (bf16*)out, H);           \
+  } while (0)
+  if (vec && H <= 1024) TL_LN(1);
+  else if (vec && H <= 2048) TL_LN(2);
+  else if (vec && H <= 4096) TL_LN(4);
+  else if (vec) TL_LN(8);
+  else if (f32) layernorm_kernel<float><<<n, 256, 0, st>>>(z, bias, w, eps, x, (float*)out, H);
+  else layernorm_kernel<bf16><<<n, 256, 0, st>>>(z, bias, w, eps, x, (bf16*)out, H);
+#undef TL_LN
+  TL_LAUNCH_CHECK("layernorm");
+  return 0;
+}
+
+int tl_cast_rows(const float* x, long long total, void* out, hipStream_t st) {
+  TL_REQUIRE(total >= 0 && (total + 255) / 256 < 2147483647LL, "cast_rows: bad size %lld", total);
+  if (total == 0) return 0;
+  cast_rows_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, (size_t)total, (bf16*)out);
+  TL_LAUNCH_CHECK("cast_rows");
+  return 0;
+}
+
+int tl_act_mul(const float* gu, int n, int I, int act, void* out, int out_dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && I > 0, "act_mul: bad sizes n=%d I=%d", n, I);
+  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH, "act_mul: no function of code %d", act);
+  if (n == 0) return 0;
+  if (out_dt == DT_F32)
+    act_mul_kernel<float><<<n, 256, 0, st>>>(gu, I, act, (float*)out);
+  else if (out_dt == DT_BF16)
+    act_mul_kernel<bf16><<<n, 256, 0, st>>>(gu, I, act, (bf16*)out);
+  else
+    TL_REQUIRE(false, "act_mul: unknown dtype code %d", out_dt);
+  TL_LAUNCH_CHECK("act_mul");
   return 0;
 }
 

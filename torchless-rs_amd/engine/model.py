@@ -90,6 +90,12 @@ class Model:
             s = mixer.state_request()
             if s is not None:
                 st[i] = s
+        # a run that reads another's keys may look further back than their owner does: the owner
+        # then keeps as many positions as its farthest reader needs
+        for i, run in enumerate(self.spec.schedule):
+            reach = getattr(self.blocks[run.layer].mixer, "kv_reach", None)
+            if run.kv_from is not None and run.kv_from in kv and reach is not None:
+                kv[run.kv_from] = kv[run.kv_from].covering(reach())
         return kv, st
 
     def make_cache(self, max_tokens: int, max_slots: Optional[int] = None, allocate: bool = True) -> Cache:

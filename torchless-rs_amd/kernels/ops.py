@@ -291,6 +291,168 @@ def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().tl_silu_mul_pairs(_p(gu), n, I2 // 2, _p(out), _stream()))
 
 
+def layernorm(z: torch.Tensor, w: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
+              add_to: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None) -> None:
+    """Layer norm with a weight and no bias of its own, y = (z - mean) / sqrt(var + eps) * w over
+    z float32 [n, H] (`bias`: added to z first, the bias of the product that made z).  Without
+    `add_to`, y goes to `out` (float32 or the compute dtype).  With it, the stream add_to += y,
+    and `out`, if given, receives the new stream in its dtype."""
+    n, H = z.shape
+    _req(z, "layernorm.z", torch.float32)
+    _req(w, "layernorm.w", torch.float32, (H,))
+    if bias is not None:
+        _req(bias, "layernorm.bias", torch.float32, (H,))
+    if add_to is not None:
+        _req(add_to, "layernorm.add_to", torch.float32, (n, H))
+    elif out is None:
+        raise KernelError("layernorm: needs `out` or `add_to`")
+    if out is not None:
+        _req(out, "layernorm.out", None, (n, H))
+    _check(lib().tl_layernorm(_p(z), _p(bias), _p(w), ctypes.c_float(eps), _p(add_to), _p(out),
+                              _code(out.dtype) if out is not None else DT_F32, n, H, _stream()))
+
+
+def cast_rows(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out = x rounded to bfloat16 (x float32, same shape)."""
+    _req(x, "cast_rows.x", torch.float32)
+    _req(out, "cast_rows.out", torch.bfloat16, tuple(x.shape))
+    _check(lib().tl_cast_rows(_p(x), ctypes.c_longlong(x.numel()), _p(out), _stream()))
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def act_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """out[n, i] = act(gu[n, i]) * gu[n, I + i]; act: silu, or gelu_tanh, the tanh form of gelu."""
+    n, I2 = gu.shape
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"act_mul: no function {activation!r}; there are {sorted(ACTIVATIONS)}")
+    _req(gu, "act_mul.gu", torch.float32)
+    _req(out, "act_mul.out", None, (n, I2 // 2))
+    _check(lib().tl_act_mul(_p(gu), n, I2 // 2, ACTIVATIONS[activation], _p(out), _code(out.dtype), _stream()))
+
+
+class ScoreTerms:
+    """What an attention adds to q.k * scale: `slopes` (float32 [nq] or None), a bias
+    -slope[h] * (p - j) by the distance of query and key; `sinks` (float32 [nq] or None), a score
+    per head with no key and no value that takes part in the softmax's sum once; `window`."""
+
+    def __init__(self, scale: float, window: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
+                 sinks: Optional[torch.Tensor] = None):
+        self.scale, self.window, self.slopes, self.sinks = float(scale), (int(window) if window else None), slopes, sinks
+
+
+def _req_pages(pages: torch.Tensor, nkv: int, dk: int, dv: int, what: str) -> None:
+    _req(pages, what + ".pages")
+    per_page = pages.numel() // pages.shape[0] if pages.shape[0] else 0
+    if pages.dim() < 2 or per_page != nkv * PAGE * (dk + dv):
+        raise KernelError(f"{what}.pages: shape {tuple(pages.shape)}, kernel needs {nkv * PAGE * (dk + dv)} "
+                          f"elements a page ({nkv} KV heads of {PAGE} keys of {dk} and values of {dv})")
+
+
+def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pages: int, row_seq, row_pos,
+                      cu_seqlens, n_cached, terms: ScoreTerms, gate, out) -> None:
+    """Attention of every row over its sequence's cached keys (j < n_cached) and this step's
+    (k_new [n, nkv, dk], v_new [n, nkv, dv]; None when everything is in the pages), causal, with
+    the terms of `ScoreTerms`; `gate` (float32 [n, nq] or None) multiplies each head's output.
+    One wave per (row, head), float32 sums."""
+    n, nq, dk = q.shape
+    B = n_cached.shape[0]
+    _req(q, "attn_scored.q", pages.dtype)
+    if k_new is not None:
+        _req(k_new, "attn_scored.k_new", pages.dtype, (n, nkv, dk))
+        _req(v_new, "attn_scored.v_new", pages.dtype, (n, nkv, dv))
+    _req_pages(pages, nkv, dk, dv, "attn_scored")
+    _req(table, "attn_scored.table", torch.int32)
+    _req(row_seq, "attn_scored.row_seq", torch.int32, (n,))
+    _req(row_pos, "attn_scored.row_pos", torch.int32, (n,))
+    _req(cu_seqlens, "attn_scored.cu_seqlens", torch.int32, (B + 1,))
+    _req(n_cached, "attn_scored.n_cached", torch.int32, (B,))
+    _req(out, "attn_scored.out", pages.dtype, (n, nq, dv))
+    if terms.slopes is not None:
+        _req(terms.slopes, "attn_scored.slopes", torch.float32, (nq,))
+    if terms.sinks is not None:
+        _req(terms.sinks, "attn_scored.sinks", torch.float32, (nq,))
+    if gate is not None:
+        _req(gate, "attn_scored.gate", torch.float32, (n, nq))
+    if table.dim() != 2 or table.shape[0] != B:
+        raise KernelError("attn_scored.table: needs one row per sequence")
+    _check(lib().tl_attn_scored_plain(_p(q), _p(k_new), _p(v_new), _p(pages), _code(q.dtype), _p(table),
+                                      table.shape[1], ring_pages, _p(row_seq), _p(row_pos), _p(cu_seqlens),
+                                      _p(n_cached), n, nq, nkv, dk, dv, int(terms.window or 0),
+                                      ctypes.c_float(terms.scale), _p(terms.slopes), _p(terms.sinks), _p(gate),
+                                      _p(out), _stream()))
+
+
+def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pages: int, ctx, n_cached,
+                     terms: ScoreTerms, gate, out) -> None:
+    """Attention with the terms of `ScoreTerms` for a step's rows: keys j < n_cached[b] from the
+    pages, later ones from this step's rows (`k_new`/`v_new`; None when everything is in the
+    pages)."""
+    attn_scored_plain(q, k_new, v_new, pages, nkv, dv, table, ring_pages, ctx.row_seq, ctx.row_pos,
+                      ctx.cu_seqlens, n_cached, terms, gate, out)
+
+
+class ProjectionTerms:
+    """What happens to a row of the fused projection [q | k | v | g] before attention: `bias`
+    (float32 over the whole row, or None); `q_norm`, `k_norm` (float32 weights over ALL of q and
+    ALL of k, or None): division by the root mean square of the whole projection, eps inside the
+    root; `temperature` (coef, every) or None: q times 1 + coef * ln(floor((p + 1) / every) + 1)."""
+
+    def __init__(self, bias=None, q_norm=None, k_norm=None, eps: float = 0.0, temperature=None):
+        self.bias, self.q_norm, self.k_norm, self.eps = bias, q_norm, k_norm, float(eps)
+        self.coef, self.every = (float(temperature[0]), float(temperature[1])) if temperature else (0.0, 1.0)
+
+
+def split_projection(proj: torch.Tensor, row_pos, terms: ProjectionTerms, nq: int, nkv: int, dk: int, dv: int,
+                     ng: int, q: torch.Tensor, k, v, gate, table=None, ring_pages: int = 0, pages=None) -> None:
+    """proj float32 [n, nq*dk + nkv*(dk+dv) + ng] -> q [n, nq, dk], gate float32 [n, ng] (after the
+    logistic function) and, with nkv > 0, k [n, nkv, dk] and v [n, nkv, dv], or, with `pages`
+    (one token a sequence, row n belongs to sequence n), k and v straight into the page of the
+    row's position."""
+    n = proj.shape[0]
+    width = nq * dk + nkv * (dk + dv) + ng
+    _req(proj, "split_projection.proj", torch.float32, (n, width))
+    _req(row_pos, "split_projection.row_pos", torch.int32, (n,))
+    _req(q, "split_projection.q", None, (n, nq, dk))
+    for t, name, size in ((terms.bias, "bias", width), (terms.q_norm, "q_norm", nq * dk), (terms.k_norm, "k_norm", nkv * dk)):
+        if t is not None:
+            _req(t, "split_projection." + name, torch.float32, (size,))
+    if ng:
+        _req(gate, "split_projection.gate", torch.float32, (n, ng))
+    if nkv and pages is None:
+        _req(k, "split_projection.k", q.dtype, (n, nkv, dk))
+        _req(v, "split_projection.v", q.dtype, (n, nkv, dv))
+    stride = 0
+    if pages is not None:
+        _req_pages(pages, nkv, dk, dv, "split_projection")
+        _req(table, "split_projection.table", torch.int32)
+        if pages.dtype != q.dtype or table.dim() != 2 or table.shape[0] != n:
+            raise KernelError("split_projection: pages of q's dtype and a page table with one row per row")
+        stride = table.shape[1]
+    _check(lib().tl_split_projection(_p(proj), _p(row_pos), _p(terms.bias), _p(terms.q_norm), _p(terms.k_norm),
+                                     ctypes.c_float(terms.eps), ctypes.c_float(terms.coef), ctypes.c_float(terms.every),
+                                     n, nq, nkv, dk, dv, ng, _p(q), _p(k), _p(v), _p(gate), _code(q.dtype),
+                                     _p(table), stride, int(ring_pages), _p(pages), _stream()))
+
+
+def kv_commit_wide(k: torch.Tensor, v: torch.Tensor, row_seq, row_pos, len_after, table: torch.Tensor,
+                   ring_pages: int, pages: torch.Tensor) -> None:
+    """Rows of keys [n, nkv, dk] and values [n, nkv, dv] into the pages of their positions (values
+    transposed, as the pages keep them); dk and dv need not be equal."""
+    n, nkv, dk = k.shape
+    dv = v.shape[2]
+    _req(k, "kv_commit_wide.k", pages.dtype)
+    _req(v, "kv_commit_wide.v", pages.dtype, (n, nkv, dv))
+    _req_pages(pages, nkv, dk, dv, "kv_commit_wide")
+    _req(row_seq, "kv_commit_wide.row_seq", torch.int32, (n,))
+    _req(row_pos, "kv_commit_wide.row_pos", torch.int32, (n,))
+    _req(table, "kv_commit_wide.table", torch.int32)
+    _req(len_after, "kv_commit_wide.len_after", torch.int32, (table.shape[0],))
+    _check(lib().tl_kv_commit_wide(_p(k), _p(v), _code(k.dtype), _p(row_seq), _p(row_pos), _p(len_after), _p(table),
+                                   table.shape[1], ring_pages, n, nkv, dk, dv, _p(pages), _stream()))
+
+
 def take_tokens(src: torch.Tensor, idx: torch.Tensor, vocab: int, tokens: torch.Tensor) -> None:
     """tokens[j] = src[idx[j]] (int32, on the device); ids outside [0, vocab) become 0."""
     n = tokens.shape[0]

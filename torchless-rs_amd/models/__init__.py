@@ -4,6 +4,7 @@ from ..config.base import ModelConfig, get_architecture
 from ..parts import base as _parts_base
 from .. import parts as _parts            # registers the parts
 from . import mistral as _mistral         # registers MistralForCausalLM
+from . import sozetar as _sozetar         # registers Sozetar
 
 
 def model_spec_for(cfg: ModelConfig):

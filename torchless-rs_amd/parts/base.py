@@ -60,9 +60,9 @@ def make_part(category: str, spec: PartSpec):
 class LayerSpec:
     prefix: str                       # the layer's tensors are named prefix + local name
     mixer: PartSpec
-    ffn: PartSpec
+    ffn: Optional[PartSpec]           # None: a layer without a feed-forward (blocks that allow it)
     mixer_norm: PartSpec
-    ffn_norm: PartSpec
+    ffn_norm: Optional[PartSpec]
     block: PartSpec = field(default_factory=lambda: PartSpec("pre_norm"))
 
 
@@ -153,6 +153,23 @@ class Norm(Part):
         on the results of the product that reads it).  None: the norm always runs by itself."""
         return None
 
+    def add_to(self, ctx: "StepContext", z: torch.Tensor, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+               bias: Optional[torch.Tensor] = None) -> None:
+        """The norm of a sublayer's output: x += norm(z + bias), z float32 [n, H] (`bias`: float32
+        [H], what the sublayer's last product left to add); `out`, if given, receives the new x in
+        its dtype.  This is the plain way in three kernels; a norm with a kernel for it overrides."""
+        from ..kernels import ops
+        if bias is not None:
+            z += bias
+        y = ctx.workspace.get("norm_add_y", tuple(z.shape), torch.float32)
+        self.forward(ctx, z, y)
+        ops.add_partials(x, y.view(1, *y.shape))
+        if out is not None:
+            if out.dtype == torch.float32:
+                out.copy_(x)
+            else:
+                ops.cast_rows(x, out)
+
 
 class Position(Part):
     """A position encoding, as the attention mixer asks for it: how q and k are rotated."""
@@ -180,11 +197,18 @@ class Mixer(Part):
         """y: normed input [n, H] (compute dtype); ADD the result to x (float32 [n, H])."""
         raise NotImplementedError
 
+    # A mixer may also offer `produce(ctx, run, y, out) -> Optional[bias]`: STORE the result in
+    # `out` (float32 [n, H]) instead of adding it to the stream, for an arrangement that norms a
+    # sublayer's output before the sum.  What it returns (float32 [H] or None) is a bias that
+    # the caller still has to add to `out` (the norm's kernel does it on the way).
+
 
 class FeedForward(Part):
     def forward(self, ctx: "StepContext", y: torch.Tensor, x: torch.Tensor) -> None:
         """y: normed input [n, H]; ADD the result to x (float32 [n, H])."""
         raise NotImplementedError
+
+    # `produce(ctx, y, out) -> Optional[bias]`: as a mixer's.
 
 
 @dataclass

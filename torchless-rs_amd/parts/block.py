@@ -1,15 +1,18 @@
-"""The arrangement of a layer: x += mixer(norm(x)); x += ffn(norm(x))
-(src/model/modules/layer.rs:28-56 of the reference).  The residual stream x
-is float32; mixer and feed-forward add into it."""
+"""The arrangements of a layer.  `PreNormBlock`: x += mixer(norm(x)); x += ffn(norm(x))
+(src/model/modules/layer.rs:28-56 of the reference).  `OutputNormBlock`: the
+sublayers read the stream itself and their OUTPUT is normed before the sum,
+x += norm(mixer(x)); x += norm(ffn(x)), the feed-forward being optional.  The
+residual stream x is float32 in both."""
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
 from ..weights.binding import WeightSpec
-from .base import (LayerSpec, Part, expect_norm, make_part, part_done, read_through_norm, register_part,
-                   splittable_entry)
+from ..kernels import ops
+from .base import (LayerSpec, Part, expect_norm, flush_pending, make_part, part_done, read_through_norm,
+                   register_part, splittable_entry)
 
 
 class PreNormBlock(Part):
@@ -55,6 +58,7 @@ class PreNormBlock(Part):
         """`norm_after`: the `entry_norm` of the block that runs next, if it has one.  The three
         helpers around each part (`read_through_norm`, `expect_norm`, `part_done`) are all that
         an arrangement needs for norms cut in two around the products."""
+        ctx.host.pop("stream_copy", None)        # this block writes the stream: a copy of it goes stale
         y = ctx.workspace.get("block_y", tuple(x.shape), ctx.dtype)
         y1 = read_through_norm(ctx, self.mixer_norm, x, y)
         expect_norm(ctx, self.mixer, self.ffn_norm, self.ffn)
@@ -66,4 +70,79 @@ class PreNormBlock(Part):
         part_done(ctx, self.ffn)
 
 
+class OutputNormBlock(Part):
+    """x += norm1(mixer(x)); then, if the layer has a feed-forward, x += norm2(ffn(x)).
+
+    A sublayer reads x itself: as it is in float32, rounded to the compute dtype otherwise.  That
+    copy is made by the norm before it (`Norm.add_to` leaves the new stream in the compute dtype
+    while it adds), by a kernel of its own only at the first block.  Parts that offer `produce`
+    store their result for the norm; any other part adds into a zeroed buffer instead."""
+
+    def __init__(self, layer: LayerSpec, mixer_norm_name: str = "norm1.", ffn_norm_name: str = "norm2."):
+        self.mixer = make_part("mixer", layer.mixer)
+        self.mixer_norm = make_part("norm", layer.mixer_norm)
+        self.ffn = make_part("ffn", layer.ffn) if layer.ffn is not None else None
+        self.ffn_norm = make_part("norm", layer.ffn_norm) if layer.ffn is not None else None
+        self.n1, self.n2 = mixer_norm_name, ffn_norm_name
+        self.graph_safe = all(p.graph_safe for p in self._parts())
+
+    def _parts(self):
+        return [p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None]
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        out: Dict[str, WeightSpec] = {}
+        for k, v in self.mixer_norm.weight_specs().items():
+            out[self.n1 + k] = v
+        out.update(self.mixer.weight_specs())
+        if self.ffn is not None:
+            for k, v in self.ffn_norm.weight_specs().items():
+                out[self.n2 + k] = v
+            out.update(self.ffn.weight_specs())
+        return out
+
+    def load(self, tensors, compute_dtype) -> None:
+        def sub(prefix):
+            return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
+        self.mixer_norm.load(sub(self.n1), compute_dtype)
+        self.mixer.load(tensors, compute_dtype)
+        if self.ffn is not None:
+            self.ffn_norm.load(sub(self.n2), compute_dtype)
+            self.ffn.load(tensors, compute_dtype)
+
+    def may_capture(self, n_rows: int) -> bool:
+        return all(p.may_capture(n_rows) for p in self._parts())
+
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        return any(p.prefers_eager(n_new, len_before, device) for p in self._parts())
+
+    @staticmethod
+    def _result(ctx, part, z, *args) -> Optional[torch.Tensor]:
+        """The part's output in z; returns the bias that is still to be added."""
+        if hasattr(part, "produce"):
+            return part.produce(ctx, *args, z)
+        z.zero_()
+        ctx.norm_ahead = None
+        part.forward(ctx, *args, z)
+        flush_pending(ctx, z)
+        return None
+
+    def forward(self, ctx, run, x: torch.Tensor, norm_after=None) -> None:
+        flush_pending(ctx, x)
+        narrow = ctx.dtype != torch.float32
+        y = x
+        if narrow:
+            y = ctx.workspace.get("stream_y", tuple(x.shape), ctx.dtype)
+            if ctx.host.pop("stream_copy", None) is not y:       # nobody left the stream there yet
+                ops.cast_rows(x, y)
+        z = ctx.workspace.get("block_z", tuple(x.shape), torch.float32)
+        bias = self._result(ctx, self.mixer, z, run, y)
+        self.mixer_norm.add_to(ctx, z, x, out=y if narrow else None, bias=bias)
+        if self.ffn is not None:
+            bias = self._result(ctx, self.ffn, z, y)
+            self.ffn_norm.add_to(ctx, z, x, out=y if narrow else None, bias=bias)
+        if narrow:
+            ctx.host["stream_copy"] = y
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "output_norm", OutputNormBlock)

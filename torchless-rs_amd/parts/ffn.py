@@ -1,5 +1,7 @@
-"""SwiGLU feed-forward: down( silu(gate y) * (up y) ), silu(g) = g / (1 + e^-g)
-(src/model/modules/mlp.rs:23-45, src/kernels/mod.rs:546-548 of the reference).
+"""Gated feed-forward: down( act(gate y) * (up y) ).  With act = silu,
+silu(g) = g / (1 + e^-g), it is SwiGLU (src/model/modules/mlp.rs:23-45,
+src/kernels/mod.rs:546-548 of the reference); `activation` chooses another
+function of the gate (`ops.ACTIVATIONS`: gelu_tanh, the tanh form of gelu).
 gate and up are bound under their own names (`names`: the leaf names are
 parameters, and a checkpoint that stores gate|up as one tensor binds that one)
 and laid side by side at load so that one product serves both."""
@@ -24,7 +26,10 @@ class SwiGLU(FeedForward):
     NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", "gate_up": None}
 
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp.",
-                 names: Optional[Dict[str, Optional[str]]] = None):
+                 names: Optional[Dict[str, Optional[str]]] = None, activation: str = "silu"):
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"gated feed-forward: no activation {activation!r}; there are {sorted(ops.ACTIVATIONS)}")
+        self.activation = activation
         self.H = int(hidden_size)
         self.I = int(intermediate_size)
         self.prefix = prefix
@@ -57,11 +62,18 @@ class SwiGLU(FeedForward):
         # bfloat16 on the matrix cores: gate and up rows interleaved so that the product's
         # epilogue applies silu(gate) * up itself and writes bfloat16
         self.paired = (compute_dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and self.I % 32 == 0
-                       and self.H % 8 == 0)
+                       and self.H % 8 == 0 and self.activation == "silu")
         self.gate_up = Linear(interleave_pairs(g, u) if self.paired else torch.cat([g, u], dim=0))
         self.down = Linear(tensors[p + nm["down"]], tiled=True)
 
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
+        self.down.add_into(self._hidden(ctx, y), x, ctx, "ffn_down_parts")
+
+    def produce(self, ctx, y: torch.Tensor, out: torch.Tensor) -> None:
+        """The result stored in `out` (float32 [n, H]) instead of added to the stream."""
+        self.down(self._hidden(ctx, y), out)
+
+    def _hidden(self, ctx, y: torch.Tensor) -> torch.Tensor:
         n = y.shape[0]
         h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
         factor = take_row_factor(ctx, usable=self.paired and ops.norm_split_ok(y, self.gate_up.weight))
@@ -79,8 +91,9 @@ class SwiGLU(FeedForward):
         else:
             gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
             self.gate_up(y, gu)
-            ops.silu_mul(gu, h)
-        self.down.add_into(h, x, ctx, "ffn_down_parts")
+            ops.act_mul(gu, h, self.activation)
+        return h
 
 
 register_part("ffn", "swiglu", SwiGLU)
+register_part("ffn", "gated", SwiGLU)          # the same part under the name that fits any activation

@@ -1,5 +1,8 @@
-"""RMSNorm.  y = x / sqrt(mean(x^2) + eps) * w, in float32
-(src/kernels/mod.rs:558-568 of the reference; weight used as it is)."""
+"""Norms over a row of the stream, in float32.
+
+RMSNorm: y = x / sqrt(mean(x^2) + eps) * w (src/kernels/mod.rs:558-568 of the
+reference; weight used as it is).  LayerNorm: y = (x - mean) / sqrt(var + eps) * w
+with var the mean of the squared deviations, a weight and no bias."""
 from __future__ import annotations
 
 from typing import Dict
@@ -42,4 +45,35 @@ class RMSNorm(Norm):
         ops.rmsnorm(x, self.weight, self.eps, out)
 
 
+class LayerNorm(Norm):
+    """Mean and variance over the row; a weight, no bias.  Besides the plain `forward` it can
+    be the norm of a sublayer's OUTPUT (`add_to`): x += norm(z), in one kernel that also
+    leaves the new stream in the compute dtype for the product that reads it next."""
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float, name: str = "weight"):
+        """`name`: the weight's leaf name behind the norm's prefix ("" where the prefix is the tensor)."""
+        self.size = int(size)
+        self.eps = float(eps)
+        self.name = name
+        self.weight = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {self.name: WeightSpec((self.size,), init="ones")}
+
+    def load(self, tensors, compute_dtype) -> None:
+        self.weight = tensors[self.name].to(torch.float32).contiguous()
+
+    def forward(self, ctx, x: torch.Tensor, out: torch.Tensor) -> None:
+        flush = getattr(ctx, "pending", None)
+        if flush is not None:
+            ops.add_partials(x, flush)
+            ctx.pending = None
+        ops.layernorm(x, self.weight, self.eps, out)
+
+    def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None) -> None:
+        ops.layernorm(z, self.weight, self.eps, out, add_to=x, bias=bias)
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "layernorm", LayerNorm)

@@ -172,7 +172,9 @@ def attention_case(dtype, nq, nkv, dk, dv, cached, new, window, slopes, sinks, g
     for b in range(B):
         for i in range(pages_of[b]):
             table[b, i] = order.pop()
-    pages = torch.full((n_pages, nkv * 64 * (dk + dv)), float("nan"), dtype=dt, device="cuda")
+    # (the shape of the cache's storage: values as wide as keys lie as [K|V, kv head, 64, d])
+    shape = (n_pages, 2, nkv, 64, dk) if dk == dv else (n_pages, nkv * 64 * (dk + dv))
+    pages = torch.full(shape, float("nan"), dtype=dt, device="cuda")
     table = dev(table)
     i32 = dict(dtype=torch.int32, device="cuda")
     # the cached positions go into the pages as a step of their own would have put them
@@ -190,11 +192,14 @@ def attention_case(dtype, nq, nkv, dk, dv, cached, new, window, slopes, sinks, g
     cu = np.concatenate([[0], np.cumsum(new)])
     all_single = all(x == 1 for x in new)
     len_after = torch.tensor([c + x for c, x in zip(cached, new)], **i32)
+    offs, cols = ops.aligned_columns(cached, new)
     ctx = types.SimpleNamespace(
         row_seq=torch.tensor([r[0] for r in rows], **i32), row_pos=torch.tensor([r[1] for r in rows], **i32),
         cu_seqlens=torch.tensor(cu, **i32), len_before=torch.tensor(cached, **i32), len_after=len_after,
+        tile_off=torch.tensor(offs, **i32),
         all_single=all_single, workspace=Workspace(torch.device("cuda")), n_rows=n, n_seqs=B, dtype=dt,
-        max_new=max(new), host={"n_new": np.asarray(new, dtype=np.int64), "len_before": np.asarray(cached, dtype=np.int64)})
+        max_new=max(new), host={"n_new": np.asarray(new, dtype=np.int64), "len_before": np.asarray(cached, dtype=np.int64),
+                                "aligned_cols": cols})
     gate = torch.rand(n, nq, generator=g) if gated else None
     terms = ops.ScoreTerms(scale, window, dev(slopes.float()) if slopes is not None else None,
                            dev(sinks.float()) if sinks is not None else None)
@@ -204,8 +209,12 @@ def attention_case(dtype, nq, nkv, dk, dv, cached, new, window, slopes, sinks, g
         ops.attention_scored(q, None, None, pages, nkv, dv, table, ring, ctx, len_after, terms,
                              dev(gate) if gated else None, out)
     else:
+        vt = None
+        if ops.scored_on_matrix_cores(dt, dk, dv):        # the matrix cores read the step's values along the keys
+            vt = torch.full((nkv, dv, cols), float("nan"), dtype=dt, device="cuda")
+            ops.v_tiles_rows(v_new, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, len_after)
         ops.attention_scored(q, k_new, v_new, pages, nkv, dv, table, ring, ctx, ctx.len_before, terms,
-                             dev(gate) if gated else None, out)
+                             dev(gate) if gated else None, out, vt_new=vt)
     want = torch.cat([plain.attend(seqs[b][0].double(), seqs[b][1].double(), seqs[b][2].double(), scale,
                                    slopes, sinks, window)[cached[b]:] for b in range(B)])
     if gated:
@@ -218,7 +227,8 @@ ATT_TOL = {"float32": 2e-5, "bfloat16": 1.2e-2}
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("what", ["nothing", "slopes", "sink", "window", "gate", "all"])
-@pytest.mark.parametrize("nq, nkv, dk, dv", [(4, 2, 16, 32), (6, 3, 40, 24), (8, 2, 64, 64), (4, 1, 32, 64), (1, 1, 8, 8)])
+@pytest.mark.parametrize("nq, nkv, dk, dv", [(4, 2, 16, 32), (6, 3, 40, 24), (8, 2, 64, 64), (4, 1, 32, 64), (1, 1, 8, 8),
+                                             (6, 1, 48, 48), (20, 1, 128, 128), (3, 3, 80, 80)])
 def test_attention_terms_one_by_one(dtype, what, nq, nkv, dk, dv):
     slopes = plain.head_slopes(nq) if what in ("slopes", "all") else None
     sinks = torch.linspace(-1, 2, nq, dtype=torch.float64) if what in ("sink", "all") else None
@@ -228,6 +238,24 @@ def test_attention_terms_one_by_one(dtype, what, nq, nkv, dk, dv):
     for cached, new in (([0, 0], [70, 9]), ([64, 3, 130], [5, 66, 2]), ([5, 64, 199], [1, 1, 1])):
         got, want = attention_case(dtype, nq, nkv, dk, dv, cached, new, window, slopes, sinks, gated, seed=len(what))
         assert rel_err(got, want) < ATT_TOL[dtype], (what, cached, new)
+
+
+def test_the_matrix_cores_serve_the_shapes_they_take(monkeypatch):
+    """bfloat16 with values as wide as keys and head sizes in steps of 16 never reaches the plain kernel,
+    in prompts, in portions after cached positions and in single-token steps; other shapes always do."""
+    from torchless_rs_amd.kernels import ops
+    calls = []
+    plain_kernel = ops.attn_scored_plain
+    monkeypatch.setattr(ops, "attn_scored_plain", lambda *a, **k: (calls.append(1), plain_kernel(*a, **k)))
+    sinks = torch.zeros(4, dtype=torch.float64)
+    for cached, new in (([0, 0], [70, 9]), ([64, 3], [5, 66]), ([5, 64, 199], [1, 1, 1])):
+        for dk in (16, 48, 128):
+            attention_case("bfloat16", 4, 2, dk, dk, cached, new, 37, plain.head_slopes(4), sinks, True, seed=1)
+        assert not calls
+    attention_case("bfloat16", 4, 2, 16, 32, [3], [5], None, None, sinks, False, seed=1)
+    attention_case("bfloat16", 4, 2, 24, 24, [3], [1], None, None, sinks, False, seed=1)
+    attention_case("float32", 4, 2, 16, 16, [3], [5], None, None, sinks, False, seed=1)
+    assert len(calls) == 3
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

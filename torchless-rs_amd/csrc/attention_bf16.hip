@@ -33,6 +33,18 @@ __device__ __forceinline__ bf16x8 z8() {
   return z;
 }
 
+// More terms on a score than q.k * scale (the TERMS variants of the kernels below; each
+// pointer may be null): slopes[h], a bias -slope * (p - j) by the distance of query and key;
+// sinks[h], a score with no key and no value that counts once in the softmax's sum; gate[row, h],
+// a factor on the head's output.  With TERMS the weights of the softmax also reach the second
+// product in two bfloat16 terms, w = hi + lo (two MFMAs), so that the product with the values
+// carries 16 bits of a weight's mantissa instead of 8.
+struct MoreTerms {
+  const float* slopes;
+  const float* sinks;
+  const float* gate;
+};
+
 // ------------------------------------------------------------------ prefill --
 // One workgroup: 128 consecutive new rows of one sequence (4 waves x 32) and
 // one query head.  Keys go by tiles of 64 positions (aligned to 64, so a tile
@@ -44,7 +56,7 @@ __device__ __forceinline__ bf16x8 z8() {
 constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
 constexpr int PF_PART_HEAD = 4;       // floats before O in a half block's partial result: maximum, sum, two of padding
 
-template <int DPAD, bool LEAN>       // LEAN (d == DPAD, 256 % (DPAD / 8) == 0): whole tiles are fetched the short way
+template <int DPAD, bool LEAN, bool TERMS = false>   // LEAN (d == DPAD, 256 % (DPAD / 8) == 0): whole tiles are fetched the short way
 __global__ void __launch_bounds__(256, DPAD <= 128 ? 2 : 1)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
@@ -52,7 +64,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     int ring_pages, const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
                     const int* __restrict__ n_cached, int B, int n_tiles, int nq, int nkv, int d,
                     int window, float scale, bf16* __restrict__ out, const int4* __restrict__ items,
-                    float* __restrict__ part, int part_ways) {
+                    float* __restrict__ part, int part_ways, MoreTerms terms) {
   constexpr int KB = DPAD / 16, VB = DPAD / 32, KLD = DPAD + 8, CH = DPAD / 8;
   constexpr int PT = DPAD / 32;        // 16-byte chunks of keys, and of values, per thread and tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -136,6 +148,15 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[vb][r] = 0.f;
   float m = -INFINITY, l = 0.f;
+  float slope = 0.f;
+  if constexpr (TERMS) {
+    if (terms.sinks != nullptr && (ways == 0 || slot == 0)) {     // the sink opens the sums, once for a row
+      m = terms.sinks[h];
+      l = 1.f;
+    }
+    if (terms.slopes != nullptr) slope = terms.slopes[h];
+  }
+  const float sc = TERMS ? 1.f : scale;       // with TERMS the scores are scaled where the bias is added
 
   const int p_lo = p_first + qt0, p_hi = p_first + min(qt0 + PF_BM, n_new) - 1;
   const int pw_lo = p_lo + wave * 32, pw_hi = min(p_hi, pw_lo + 31);    // this wave's positions
@@ -285,6 +306,15 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     __builtin_amdgcn_s_setprio(0);
     // s[nb][r] = k.q of key j0 + 32 nb + 8 (r/4) + 4 half + r%4 with this lane's query.
     // Only tiles that cross the wave's causal edge, the window's edge or the rows' end need masks.
+    if constexpr (TERMS) {
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+          s[nb][r] = s[nb][r] * scale - slope * (float)(p_me - j);
+        }
+    }
     const bool edge = j0 + PF_BN - 1 > pw_lo || (window > 0 && j0 <= pw_hi - window) ||
                       pw_lo + 31 > pw_hi;
     if (edge) {
@@ -303,7 +333,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 #pragma unroll
       for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-    const float m_new = fmaxf(m, tmax * scale);          // scale > 0: the maximum of the scaled scores
+    const float m_new = fmaxf(m, tmax * sc);             // scale > 0: the maximum of the scaled scores
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
     if (__ballot(m_new != m) != 0ull) {                  // the running maximum moved in some lane
       const float alpha = __expf(m - m_use);
@@ -315,15 +345,18 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
       m = m_new;
     }
     // p = exp(s * scale - m) = 2^(s * c1 + c0)
-    const float c1 = scale * 1.44269504088896f, c0 = -m_use * 1.44269504088896f;
+    const float c1 = sc * 1.44269504088896f, c0 = -m_use * 1.44269504088896f;
     float psum = 0.f;
     bf16x8 pb[2][2];
+    bf16x8 pb_lo[TERMS ? 2 : 1][2];       // what the rounding of a weight to bfloat16 left over
     // probability e of the tile's 32 (e = 16 nb + r), in the order of the sum
     auto soft = [&](int e) {
       const int nb = e / 16, r = e % 16;
       const float pv = __builtin_amdgcn_exp2f(fmaf(s[nb][r], c1, c0));
       psum += pv;
-      pb[nb][r / 8][r % 8] = (bf16)pv;
+      const bf16 hi = (bf16)pv;
+      pb[nb][r / 8][r % 8] = hi;
+      if constexpr (TERMS) pb_lo[nb][r / 8][r % 8] = (bf16)(pv - (float)hi);
     };
     // values of block vb against probabilities 8 qd .. 8 qd + 7 (qd = 2 nb + mm): these are keys
     // kk + {0..3} and kk + 8 + {0..3}, kk = 32 nb + 16 mm + 4 half
@@ -348,7 +381,13 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     for (int qd = 0; qd < 4; ++qd) {
 #pragma unroll
       for (int vb = 0; vb < VB; ++vb) {
-        o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(qd, vb), pb[qd / 2][qd % 2], o[vb], 0, 0, 0);
+        if constexpr (TERMS) {
+          const bf16x8 va = vfrag(qd, vb);
+          o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[qd / 2][qd % 2], o[vb], 0, 0, 0);
+          o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb_lo[qd / 2][qd % 2], o[vb], 0, 0, 0);
+        } else {
+          o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(qd, vb), pb[qd / 2][qd % 2], o[vb], 0, 0, 0);
+        }
         if (qd < 3) {
 #pragma unroll
           for (int e = (8 * vb) / VB; e < (8 * (vb + 1)) / VB; ++e) soft(8 * (qd + 1) + e);
@@ -381,7 +420,9 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   }
   if (q_ok) {
     bf16* op = out + ((size_t)(row0 + qr) * nq + h) * d;
-    const float inv = 1.0f / l;
+    float inv = 1.0f / l;
+    if constexpr (TERMS)
+      if (terms.gate != nullptr) inv *= terms.gate[(size_t)(row0 + qr) * nq + h];
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb)
 #pragma unroll
@@ -440,12 +481,13 @@ attn_prefill_merge_kernel(const float* __restrict__ part, int part_ways, const i
 // result is written at once.
 constexpr int DC_WAVES = 4;
 
-template <int DPAD, bool LEAN>   // DPAD: multiple of 32; LEAN: d == DPAD, loads without guards at fixed offsets
+template <int DPAD, bool LEAN, bool TERMS = false>   // DPAD: multiple of 32; LEAN: d == DPAD, loads without guards at fixed offsets
 __global__ void __launch_bounds__(DC_WAVES * 64)
 attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                    const int* __restrict__ table, int table_stride, int ring_pages,
                    const int* __restrict__ row_pos, int nq, int nkv, int d, int window, float scale,
-                   int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out) {
+                   int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out,
+                   MoreTerms terms) {
   constexpr int KB = DPAD / 32, VB = DPAD / 16;
   constexpr bool APART = DPAD <= 128;        // room in LDS for every wave's scaled O^T: one barrier instead of four
   __shared__ float red_o[(APART ? DC_WAVES : 1) * VB * 4 * 64];
@@ -480,6 +522,9 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 #pragma unroll
   for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
+  float slope = 0.f;
+  if constexpr (TERMS)
+    if (terms.slopes != nullptr) slope = terms.slopes[h];
 
   // the split's groups of 32 keys go round the waves; a wave's pages are two apart, and the id of
   // its next page is looked up while it works on this one
@@ -546,7 +591,8 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       for (int e = 0; e < 8; ++e) {
         const int j = j0 + 8 * kg + e;
         const bool ok = j <= p && j >= lo;
-        sv[e] = ok ? s[e / 4][e % 4] * scale : -INFINITY;
+        if constexpr (TERMS) sv[e] = ok ? s[e / 4][e % 4] * scale - slope * (float)(p - j) : -INFINITY;
+        else sv[e] = ok ? s[e / 4][e % 4] * scale : -INFINITY;
         tmax = fmaxf(tmax, sv[e]);
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
@@ -554,12 +600,13 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       const float m_new = fmaxf(m, tmax);              // finite: the group holds a visible key
       const float alpha = __expf(m - m_new);
       float psum = 0.f;
-      bf16x8 pb;
+      bf16x8 pb, pb_lo;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float pv = __expf(sv[e] - m_new);
         psum += pv;
         pb[e] = (bf16)pv;
+        if constexpr (TERMS) pb_lo[e] = (bf16)(pv - (float)pb[e]);
       }
       psum += __shfl_xor(psum, 16, WAVE);
       psum += __shfl_xor(psum, 32, WAVE);
@@ -583,7 +630,10 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
           for (int r = 0; r < 4; ++r) o[vb][r] *= alpha;
       }
 #pragma unroll
-      for (int vb = 0; vb < VB; ++vb) o[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[vb], pb, o[vb], 0, 0, 0);
+      for (int vb = 0; vb < VB; ++vb) {
+        o[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[vb], pb, o[vb], 0, 0, 0);
+        if constexpr (TERMS) o[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[vb], pb_lo, o[vb], 0, 0, 0);
+      }
     }
   }
   // o[vb][r] = O[dv = 16 vb + 4 kg + r][head li]; m, l are per head li (equal in the 4 kg lanes).
@@ -640,12 +690,25 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
     }
     const int idx = ((dv / 16) * 4 + (dv % 4)) * 64 + ((dv % 16) / 4) * 16 + hd;
     const size_t bh = (size_t)b * nq + kvh * g + hg * 16 + hd;
+    float fs = 1.f;                                     // what the sink leaves of this split's sums
+    if constexpr (TERMS) {
+      if (terms.sinks != nullptr && split == 0) {       // the sink counts once: with the first split
+        const float sk = terms.sinks[kvh * g + hg * 16 + hd];
+        const float ms = fmaxf(mh, sk);
+        fs = (mh == -INFINITY) ? 0.f : __expf(mh - ms);
+        ll = ll * fs + __expf(sk - ms);
+        mh = ms;
+      }
+    }
     if (n_splits == 1) {                                // nothing to merge with
-      out[bh * d + dv] = (bf16)(o_sum(idx) / ll);
+      float res = o_sum(idx) * fs / ll;
+      if constexpr (TERMS)
+        if (terms.gate != nullptr) res *= terms.gate[bh];
+      out[bh * d + dv] = (bf16)res;
       continue;
     }
     float* dst = part + (bh * n_splits + split) * (d + 2);
-    dst[2 + dv] = o_sum(idx);
+    dst[2 + dv] = o_sum(idx) * fs;
     if (dv == 0) {
       dst[0] = mh;
       dst[1] = ll;
@@ -875,7 +938,8 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
 // this lane's elements) issued together, so that a usual split count costs one trip to memory;
 // chunks merge by the running-maximum rule.
 __global__ void __launch_bounds__(64)
-attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, bf16* __restrict__ out) {
+attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, bf16* __restrict__ out,
+                           const float* __restrict__ gate = nullptr) {
   constexpr int CH = 8, MAXV = 4;                      // d <= 256: at most 4 elements a lane
   const size_t bh = blockIdx.x;
   const float* src = part + bh * n_splits * (d + 2);
@@ -912,27 +976,28 @@ attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, 
     }
     mm = mc;
   }
+  const float gt = gate != nullptr ? gate[bh] : 1.f;       // a factor on the head's output (or none)
 #pragma unroll
   for (int v = 0; v < MAXV; ++v)
-    if (lane + 64 * v < d) out[bh * d + lane + 64 * v] = (bf16)(acc[v] / ll);
+    if (lane + 64 * v < d) out[bh * d + lane + 64 * v] = (bf16)(acc[v] / ll * gt);
 }
 
-template <int DPAD>
-static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, int vt_cols,
+template <int DPAD, bool TERMS>
+static int launch_prefill_v(const bf16* q, const bf16* k_new, const bf16* vt_new, int vt_cols,
                           const int* tile_off, const bf16* pages, const int* table, int table_stride, int ring_pages, const int* row_pos,
                           const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
                           int d, int window, float scale, bf16* out, const int4* items, const int4* cut_blocks,
-                          int n_cut, float* part, int part_ways, hipStream_t st) {
+                          int n_cut, float* part, int part_ways, hipStream_t st, MoreTerms terms) {
   const size_t smem = ((size_t)PF_BN * (DPAD + 8) + (size_t)DPAD * PF_VLD) * sizeof(bf16);
   constexpr bool can_lean = 256 % (DPAD / 8) == 0;
   if (smem > 48 * 1024) {
     static bool raised = false;
     if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, false>),
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, false, TERMS>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
       if constexpr (can_lean)
         if (e == hipSuccess)
-          e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, true>),
+          e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, true, TERMS>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
       if (e != hipSuccess) {
         set_error("attn_prefill: cannot have %zu bytes of LDS: %s", smem, hipGetErrorString(e));
@@ -948,15 +1013,15 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
   }
   const unsigned grid = (unsigned)total;
   if (can_lean && d == DPAD)
-    attn_prefill_kernel<DPAD, can_lean><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+    attn_prefill_kernel<DPAD, can_lean, TERMS><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                              table_stride, ring_pages, row_pos, cu_seqlens,
                                                              n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
-                                                             items, part, part_ways);
+                                                             items, part, part_ways, terms);
   else
-    attn_prefill_kernel<DPAD, false><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+    attn_prefill_kernel<DPAD, false, TERMS><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                               table_stride, ring_pages, row_pos, cu_seqlens,
                                                               n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
-                                                              items, part, part_ways);
+                                                              items, part, part_ways, terms);
   TL_LAUNCH_CHECK("attn_prefill");
   if (n_cut > 0) {
     const int pieces = (PF_BM * d + PF_MERGE - 1) / PF_MERGE;
@@ -967,6 +1032,23 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
   return 0;
 }
 
+// terms null: the plain scores; else the TERMS variant of the kernel (a kernel of its own, so that
+// the plain one keeps its registers)
+template <int DPAD>
+static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, int vt_cols,
+                          const int* tile_off, const bf16* pages, const int* table, int table_stride, int ring_pages, const int* row_pos,
+                          const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
+                          int d, int window, float scale, bf16* out, const int4* items, const int4* cut_blocks,
+                          int n_cut, float* part, int part_ways, hipStream_t st, const MoreTerms* terms) {
+  if (terms != nullptr)
+    return launch_prefill_v<DPAD, true>(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages,
+                                        row_pos, cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
+                                        items, cut_blocks, n_cut, part, part_ways, st, *terms);
+  return launch_prefill_v<DPAD, false>(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages,
+                                       row_pos, cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
+                                       items, cut_blocks, n_cut, part, part_ways, st, MoreTerms{});
+}
+
 // which decode kernel serves head sizes 64, 128 and 256 (tests and measurements may switch)
 static bool decode_through_lds = true;
 constexpr int DR_MAX_PAGES = 2048;      // most pages of a sequence that the kernel through LDS keeps the ids of (8 KB)
@@ -974,9 +1056,25 @@ constexpr int DR_MAX_PAGES = 2048;      // most pages of a sequence that the ker
 template <int DPAD>
 static int launch_decode(const bf16* q, const bf16* pages, const int* table, int table_stride,
                          int ring_pages, const int* row_pos, int B, int nq, int nkv, int d, int window,
-                         float scale, int n_splits, float* part, bf16* out, hipStream_t st) {
+                         float scale, int n_splits, float* part, bf16* out, hipStream_t st, const MoreTerms* terms) {
   const int g = nq / nkv, head_groups = (g + 15) / 16;
   dim3 grid(B * nkv * head_groups, n_splits);
+  if (terms != nullptr) {         // more terms on the scores: the kernel that reads the pages into registers
+    if (d == DPAD)
+      attn_decode_kernel<DPAD, true, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                            row_pos, nq, nkv, d, window, scale, n_splits,
+                                                                            head_groups, part, out, *terms);
+    else
+      attn_decode_kernel<DPAD, false, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                             row_pos, nq, nkv, d, window, scale, n_splits,
+                                                                             head_groups, part, out, *terms);
+    TL_LAUNCH_CHECK("attn_decode with terms");
+    if (n_splits > 1) {
+      attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out, terms->gate);
+      TL_LAUNCH_CHECK("attn_decode_combine");
+    }
+    return 0;
+  }
   if constexpr (DPAD == 64 || DPAD == 128 || DPAD == 256) {
     if (d == DPAD && decode_through_lds && table_stride <= DR_MAX_PAGES) {
       constexpr int NS = DPAD == 64 ? 4 : 2;         // 64 KB of LDS, two workgroups a compute unit; heads of 256: 128 KB, one
@@ -1005,11 +1103,11 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
   if (d == DPAD)
     attn_decode_kernel<DPAD, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
                                                                     row_pos, nq, nkv, d, window, scale, n_splits,
-                                                                    head_groups, part, out);
+                                                                    head_groups, part, out, MoreTerms{});
   else
     attn_decode_kernel<DPAD, false><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
                                                                      row_pos, nq, nkv, d, window, scale, n_splits,
-                                                                     head_groups, part, out);
+                                                                     head_groups, part, out, MoreTerms{});
   TL_LAUNCH_CHECK("attn_decode");
   if (n_splits > 1) {
     attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);
@@ -1036,13 +1134,15 @@ using namespace tl;
 
 // vt_new: this step's values transposed, [nkv][d][vt_cols]; the value of sequence b at position p
 // lies in column tile_off[b] + p - 64 * (n_cached[b] / 64); tile_off and vt_cols multiples of 64
-extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void* vt_new, int vt_cols,
+static int attn_prefill_entry(const void* q, const void* k_new, const void* vt_new, int vt_cols,
                                     const int* tile_off, const void* pages, const int* table, int table_stride,
                                     int ring_pages, const int* row_pos, const int* cu_seqlens,
                                     const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
                                     int window, float scale, void* out, const int* items, const int* cut_blocks,
                                     int n_cut, float* part, int part_ways, long long part_floats, int n_rows,
-                                    hipStream_t st) {
+                                    hipStream_t st, const MoreTerms* terms) {
+  TL_REQUIRE(terms == nullptr || (n_cut == 0 && items == nullptr), "attn_prefill: blocks whose keys are cut into "
+             "runs are merged without the gate: not with more terms");
   TL_REQUIRE(B > 0 && n_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0 && nq <= 65535,
              "attn_prefill: bad sizes B=%d tiles=%d nq=%d nkv=%d", B, n_tiles, nq, nkv);
   // items (or null): n_tiles entries laid out by the host, see the kernel; cut_blocks: the n_cut blocks
@@ -1070,8 +1170,34 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
   TL_BY_DPAD(launch_prefill, (const bf16*)q, (const bf16*)k_new, (const bf16*)vt_new, vt_cols, tile_off,
              (const bf16*)pages, table, table_stride, ring_pages, row_pos, cu_seqlens, n_cached, B,
              n_tiles, nq, nkv, d, window, scale, (bf16*)out, reinterpret_cast<const int4*>(items),
-             reinterpret_cast<const int4*>(cut_blocks), n_cut, part, part_ways, st);
+             reinterpret_cast<const int4*>(cut_blocks), n_cut, part, part_ways, st, terms);
   return 1;
+}
+
+extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void* vt_new, int vt_cols,
+                                    const int* tile_off, const void* pages, const int* table, int table_stride,
+                                    int ring_pages, const int* row_pos, const int* cu_seqlens,
+                                    const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
+                                    int window, float scale, void* out, const int* items, const int* cut_blocks,
+                                    int n_cut, float* part, int part_ways, long long part_floats, int n_rows,
+                                    hipStream_t st) {
+  return attn_prefill_entry(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages, row_pos,
+                            cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out, items, cut_blocks, n_cut,
+                            part, part_ways, part_floats, n_rows, st, nullptr);
+}
+
+// The same with more terms on the scores (each of slopes [nq], sinks [nq], gate [rows, nq] may be null):
+// see MoreTerms.  Whole blocks only (no runs of a block's keys).
+extern "C" int tl_attn_prefill_terms_bf16(const void* q, const void* k_new, const void* vt_new, int vt_cols,
+                                          const int* tile_off, const void* pages, const int* table, int table_stride,
+                                          int ring_pages, const int* row_pos, const int* cu_seqlens,
+                                          const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
+                                          int window, float scale, const float* slopes, const float* sinks,
+                                          const float* gate, void* out, hipStream_t st) {
+  const MoreTerms terms{slopes, sinks, gate};
+  return attn_prefill_entry(q, k_new, vt_new, vt_cols, tile_off, pages, table, table_stride, ring_pages, row_pos,
+                            cu_seqlens, n_cached, B, n_tiles, nq, nkv, d, window, scale, out, nullptr, nullptr, 0,
+                            nullptr, 0, 0, 0, st, &terms);
 }
 
 // For tests and measurements: 1 (the default) lets head sizes 64, 128 and 256 go through the kernel that stages the
@@ -1083,10 +1209,10 @@ extern "C" int tl_attn_decode_through_lds(int on) {
 }
 
 // part: float scratch of B * nq * n_splits * (d + 2) elements (not touched when n_splits is 1)
-extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* table, int table_stride,
+static int attn_decode_entry(const void* q, const void* pages, const int* table, int table_stride,
                                    int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
                                    int window, float scale, int n_splits, float* part, void* out,
-                                   hipStream_t st) {
+                                   hipStream_t st, const MoreTerms* terms) {
   TL_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes B=%d nq=%d nkv=%d", B,
              nq, nkv);
   TL_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attn_decode: head size %d is not served "
@@ -1095,8 +1221,26 @@ extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* 
              "attn_decode: bad geometry ring_pages=%d table_stride=%d window=%d splits=%d", ring_pages,
              table_stride, window, n_splits);
   TL_BY_DPAD(launch_decode, (const bf16*)q, (const bf16*)pages, table, table_stride, ring_pages, row_pos,
-             B, nq, nkv, d, window, scale, n_splits, part, (bf16*)out, st);
+             B, nq, nkv, d, window, scale, n_splits, part, (bf16*)out, st, terms);
   return 1;
+}
+
+extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* table, int table_stride,
+                                   int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
+                                   int window, float scale, int n_splits, float* part, void* out,
+                                   hipStream_t st) {
+  return attn_decode_entry(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale, n_splits,
+                           part, out, st, nullptr);
+}
+
+// The same with more terms on the scores (slopes [nq], sinks [nq], gate [B, nq]; each may be null)
+extern "C" int tl_attn_decode_terms_bf16(const void* q, const void* pages, const int* table, int table_stride,
+                                         int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
+                                         int window, float scale, int n_splits, float* part, const float* slopes,
+                                         const float* sinks, const float* gate, void* out, hipStream_t st) {
+  const MoreTerms terms{slopes, sinks, gate};
+  return attn_decode_entry(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale, n_splits,
+                           part, out, st, &terms);
 }
 
 // ---- the entry point that allocates nothing (declared in no_alloc.h) --------

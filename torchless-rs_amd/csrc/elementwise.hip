@@ -243,9 +243,9 @@ __device__ __forceinline__ ColumnTile column_tile(int col0, int B, const int* ti
 // vt[kv head][dv][column] = v of the row at that column, from the fused projection (float):
 // the transposed values of a step, written in whole lines (a row-by-row kernel writes them
 // two bytes at a time, a line apart).  grid: (columns / 64, kv heads, d / 64 rounded up).
-template <typename TO>
+template <typename TO, typename TS = float>       // TS: the type of the rows the values are read from
 __device__ __forceinline__ void v_tile(int col_block, int kvh, int d_block, TO (*tile)[PAGE + 2],
-                                       const float* __restrict__ qkv, int width, int v_off, int d,
+                                       const TS* __restrict__ qkv, int width, int v_off, int d,
                                        TO* __restrict__ vt, int vt_cols, int B, const int* __restrict__ cu_seqlens,
                                        const int* __restrict__ tile_off, const int* __restrict__ n_cached,
                                        const int* __restrict__ len_after) {
@@ -261,7 +261,7 @@ __device__ __forceinline__ void v_tile(int col_block, int kvh, int d_block, TO (
     const int idx = threadIdx.x + 256 * u;
     const int r = idx / dc, i = idx % dc, p = t.p0 + r;
     tmp[u] = (idx < PAGE * dc && p >= t.lo && p < t.hi)
-                 ? qkv[(size_t)(row0 + p) * width + v_off + kvh * d + c0 + i] : 0.f;
+                 ? to_f32(qkv[(size_t)(row0 + p) * width + v_off + kvh * d + c0 + i]) : 0.f;
   }
 #pragma unroll
   for (int u = 0; u < 16; ++u) {
@@ -277,13 +277,13 @@ __device__ __forceinline__ void v_tile(int col_block, int kvh, int d_block, TO (
   }
 }
 
-template <typename TO>
+template <typename TO, typename TS = float>
 __global__ void __launch_bounds__(256)
-v_tiles_kernel(const float* __restrict__ qkv, int width, int v_off, int d, TO* __restrict__ vt,
+v_tiles_kernel(const TS* __restrict__ qkv, int width, int v_off, int d, TO* __restrict__ vt,
                int vt_cols, int B, const int* __restrict__ cu_seqlens, const int* __restrict__ tile_off,
                const int* __restrict__ n_cached, const int* __restrict__ len_after) {
   __shared__ TO tile[64][PAGE + 2];
-  v_tile<TO>(blockIdx.x, blockIdx.y, blockIdx.z, tile, qkv, width, v_off, d, vt, vt_cols, B, cu_seqlens, tile_off,
+  v_tile<TO, TS>(blockIdx.x, blockIdx.y, blockIdx.z, tile, qkv, width, v_off, d, vt, vt_cols, B, cu_seqlens, tile_off,
              n_cached, len_after);
 }
 
@@ -772,6 +772,28 @@ int tl_kv_commit_tiles(const void* k, const void* vt, int vt_cols, int dt, const
 }
 
 // tl_rope_split (q and k only) and tl_v_tiles in one launch: see rope_v_tiles_kernel
+// The same from rows of values alone, v[n, nkv, d] in the type of vt (a step whose values were
+// split off the projection by another kernel)
+int tl_v_tiles_rows(const void* v, int n, int nkv, int d, void* vt, int vt_cols, int dt, int B,
+                    const int* cu_seqlens, const int* tile_off, const int* n_cached, const int* len_after,
+                    hipStream_t st) {
+  TL_REQUIRE(n >= 0 && nkv > 0 && d > 0 && B > 0, "v_tiles_rows: bad sizes n=%d nkv=%d d=%d B=%d", n, nkv, d, B);
+  TL_REQUIRE(vt_cols > 0 && vt_cols % PAGE == 0 && nkv <= 65535, "v_tiles_rows: %d columns (a multiple of 64), %d KV heads",
+             vt_cols, nkv);
+  if (n == 0) return 0;
+  const dim3 grid(vt_cols / PAGE, nkv, (d + 63) / 64);
+  if (dt == DT_F32)
+    v_tiles_kernel<float, float><<<grid, 256, 0, st>>>((const float*)v, nkv * d, 0, d, (float*)vt, vt_cols, B, cu_seqlens,
+                                                        tile_off, n_cached, len_after);
+  else if (dt == DT_BF16)
+    v_tiles_kernel<bf16, bf16><<<grid, 256, 0, st>>>((const bf16*)v, nkv * d, 0, d, (bf16*)vt, vt_cols, B, cu_seqlens,
+                                                      tile_off, n_cached, len_after);
+  else
+    TL_REQUIRE(false, "v_tiles_rows: unknown dtype code %d", dt);
+  TL_LAUNCH_CHECK("v_tiles_rows");
+  return 0;
+}
+
 int tl_rope_v_tiles(const float* qkv, const int* row_pos, const float* inv_freq, int rotary_dim, int interleaved,
                     int n, int nq, int nkv, int d, void* q, void* k, void* vt, int vt_cols, int B,
                     const int* cu_seqlens, const int* tile_off, const int* n_cached, const int* len_after, int dt,

@@ -201,6 +201,19 @@ def v_tiles(qkv: torch.Tensor, nq: int, nkv: int, d: int, vt: torch.Tensor, cu_s
                             _p(tile_off), _p(n_cached), _p(len_after), _stream()))
 
 
+def v_tiles_rows(v: torch.Tensor, vt: torch.Tensor, cu_seqlens, tile_off, n_cached, len_after) -> None:
+    """`v_tiles` from rows of values alone: v [n, nkv, d] in vt's dtype -> vt [nkv, d, columns]."""
+    n, nkv, d = v.shape
+    _req(v, "v_tiles_rows.v", vt.dtype)
+    _req(vt, "v_tiles_rows.vt")
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % PAGE:
+        raise KernelError(f"v_tiles_rows.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of {PAGE}]")
+    B = tile_off.shape[0]
+    _tiles_args(B, cu_seqlens, tile_off, n_cached, len_after, "v_tiles_rows")
+    _check(lib().tl_v_tiles_rows(_p(v), n, nkv, d, _p(vt), vt.shape[2], _code(vt.dtype), B, _p(cu_seqlens),
+                                 _p(tile_off), _p(n_cached), _p(len_after), _stream()))
+
+
 def rope_v_tiles(qkv: torch.Tensor, row_pos, rotation, nq: int, nkv: int, d: int, q: torch.Tensor, k: torch.Tensor,
                  vt: torch.Tensor, cu_seqlens, tile_off, n_cached, len_after) -> None:
     """`rope_split` (q and k) and `v_tiles` in one launch: the same bits as the two."""
@@ -384,13 +397,52 @@ def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pag
                                       _p(out), _stream()))
 
 
+def scored_on_matrix_cores(dtype: torch.dtype, dk: int, dv: int) -> bool:
+    """Does `attention_scored` run on the matrix cores (bfloat16, values as wide as keys, head sizes in
+    steps of 16)?  Steps with several rows a sequence then take their values transposed (`vt_new`)."""
+    return dtype == torch.bfloat16 and dk == dv and dk % 16 == 0 and 16 <= dk <= 256
+
+
+def _terms_args(terms: ScoreTerms, gate, n: int, nq: int):
+    if terms.slopes is not None:
+        _req(terms.slopes, "attn_scored.slopes", torch.float32, (nq,))
+    if terms.sinks is not None:
+        _req(terms.sinks, "attn_scored.sinks", torch.float32, (nq,))
+    if gate is not None:
+        _req(gate, "attn_scored.gate", torch.float32, (n, nq))
+    return _p(terms.slopes), _p(terms.sinks), _p(gate)
+
+
 def attention_scored(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pages: int, ctx, n_cached,
-                     terms: ScoreTerms, gate, out) -> None:
+                     terms: ScoreTerms, gate, out, vt_new=None) -> None:
     """Attention with the terms of `ScoreTerms` for a step's rows: keys j < n_cached[b] from the
     pages, later ones from this step's rows (`k_new`/`v_new`; None when everything is in the
-    pages)."""
-    attn_scored_plain(q, k_new, v_new, pages, nkv, dv, table, ring_pages, ctx.row_seq, ctx.row_pos,
-                      ctx.cu_seqlens, n_cached, terms, gate, out)
+    pages).  Where `scored_on_matrix_cores`, single-token steps and steps with longer rows each run
+    in the TERMS variant of the kernels of `attention` (the latter takes the step's values
+    transposed, `vt_new`); everything else in the plain kernel."""
+    n, nq, dk = q.shape
+    fast = scored_on_matrix_cores(q.dtype, dk, dv) and pages.dim() == 5
+    if fast and k_new is None and ctx.all_single:
+        splits = decode_splits(n, nq, nkv, table.shape[1], compute_units(q.device), dk)
+        part = ctx.workspace.get("attn_part", (n * nq * splits * (dk + 2),), torch.float32)
+        _decode_args(q, pages, table, ctx.row_pos, part, out, splits)
+        slopes, sinks, gt = _terms_args(terms, gate, n, nq)
+        _check(lib().tl_attn_decode_terms_bf16(_p(q), _p(pages), _p(table), table.shape[1], ring_pages, _p(ctx.row_pos),
+                                               n, nq, nkv, dk, int(terms.window or 0), ctypes.c_float(terms.scale),
+                                               int(splits), _p(part), slopes, sinks, gt, _p(out), _stream()))
+    elif fast and k_new is not None and vt_new is not None:
+        B = n_cached.shape[0]
+        n_tiles = int(sum(-(-int(x) // PREFILL_BLOCK) for x in ctx.host["n_new"]))
+        _prefill_args(q, k_new, vt_new, ctx.tile_off, pages, table, ctx.row_pos, ctx.cu_seqlens, n_cached, out)
+        slopes, sinks, gt = _terms_args(terms, gate, n, nq)
+        _check(lib().tl_attn_prefill_terms_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(ctx.tile_off), _p(pages),
+                                                _p(table), table.shape[1], ring_pages, _p(ctx.row_pos),
+                                                _p(ctx.cu_seqlens), _p(n_cached), B, n_tiles, nq, nkv, dk,
+                                                int(terms.window or 0), ctypes.c_float(terms.scale), slopes, sinks, gt,
+                                                _p(out), _stream()))
+    else:
+        attn_scored_plain(q, k_new, v_new, pages, nkv, dv, table, ring_pages, ctx.row_seq, ctx.row_pos,
+                          ctx.cu_seqlens, n_cached, terms, gate, out)
 
 
 class ProjectionTerms:
@@ -973,14 +1025,8 @@ def prefill_serves(dtype: torch.dtype, d: int) -> bool:
     return dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256
 
 
-def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int, row_pos, cu_seqlens,
-                      n_cached, n_tiles: int, window: Optional[int], scale: float, out,
-                      cuts: Optional[PrefillCuts] = None, part: Optional[torch.Tensor] = None) -> None:
-    """bfloat16 attention for steps with many rows per sequence.  `vt_new`:
-    this step's values transposed [nkv, d, cols] at the columns that
-    `aligned_columns` gives (`tile_off`).  `n_tiles`: sum over the sequences
-    of ceil(rows / 128).  `cuts` (`prefill_cuts` of this step) with `part`, float32 scratch of
-    n * nq * cuts.ways * (d + 4) elements: the keys of long blocks go to several workgroups each."""
+def _prefill_args(q, k_new, vt_new, tile_off, pages, table, row_pos, cu_seqlens, n_cached, out) -> None:
+    """The operands of the attention for steps with many rows, checked against what its grid assumes."""
     n, nq, d = q.shape
     nkv = pages.shape[2]
     B = n_cached.shape[0]
@@ -1000,6 +1046,20 @@ def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int,
     _req(out, "attn.out", torch.bfloat16, (n, nq, d))
     if table.dim() != 2 or table.shape[0] != B:
         raise KernelError("attn.table: needs one row per sequence")
+
+
+def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int, row_pos, cu_seqlens,
+                      n_cached, n_tiles: int, window: Optional[int], scale: float, out,
+                      cuts: Optional[PrefillCuts] = None, part: Optional[torch.Tensor] = None) -> None:
+    """bfloat16 attention for steps with many rows per sequence.  `vt_new`:
+    this step's values transposed [nkv, d, cols] at the columns that
+    `aligned_columns` gives (`tile_off`).  `n_tiles`: sum over the sequences
+    of ceil(rows / 128).  `cuts` (`prefill_cuts` of this step) with `part`, float32 scratch of
+    n * nq * cuts.ways * (d + 4) elements: the keys of long blocks go to several workgroups each."""
+    n, nq, d = q.shape
+    nkv = pages.shape[2]
+    B = n_cached.shape[0]
+    _prefill_args(q, k_new, vt_new, tile_off, pages, table, row_pos, cu_seqlens, n_cached, out)
     if cuts is None:
         _check(lib().tl_attn_prefill_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(tile_off), _p(pages),
                                           _p(table), table.shape[1], ring_pages, _p(row_pos), _p(cu_seqlens),
@@ -1022,11 +1082,8 @@ def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int,
                                       _p(part), cuts.ways, ctypes.c_longlong(part.numel()), n, _stream()))
 
 
-def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional[int], scale: float,
-                     n_splits: int, part, out) -> None:
-    """bfloat16 attention of one new token per sequence over its pages (the
-    token's own key is already committed).  `part`: float32 scratch of at
-    least B * nq * n_splits * (d + 2) elements."""
+def _decode_args(q, pages, table, row_pos, part, out, n_splits: int) -> None:
+    """The operands of single-token attention, checked against what its grid assumes."""
     B, nq, d = q.shape
     nkv = pages.shape[2]
     _req(q, "attn.q", torch.bfloat16)
@@ -1041,6 +1098,16 @@ def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional
         raise KernelError("attn.table: needs one row per sequence")
     if part.numel() < B * nq * n_splits * (d + 2):
         raise KernelError(f"attn.part: {part.numel()} elements, kernel needs {B * nq * n_splits * (d + 2)}")
+
+
+def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional[int], scale: float,
+                     n_splits: int, part, out) -> None:
+    """bfloat16 attention of one new token per sequence over its pages (the
+    token's own key is already committed).  `part`: float32 scratch of at
+    least B * nq * n_splits * (d + 2) elements."""
+    B, nq, d = q.shape
+    nkv = pages.shape[2]
+    _decode_args(q, pages, table, row_pos, part, out, n_splits)
     _check(lib().tl_attn_decode_bf16(_p(q), _p(pages), _p(table), table.shape[1], ring_pages, _p(row_pos),
                                      B, nq, nkv, d, int(window or 0), ctypes.c_float(scale),
                                      int(n_splits), _p(part), _p(out), _stream()))

@@ -164,7 +164,8 @@ class ScoredAttentionMixer(Mixer):
         q = ws.get("sattn_q", (n, nq, dk), ctx.dtype)
         gate = ws.get("sattn_gate", (n, ng), torch.float32) if ng else None
         att = ws.get("sattn_out", (n, nq, dv), ctx.dtype)
-        k = v = None
+        k = v = vt = None
+        tiles = ops.scored_on_matrix_cores(ctx.dtype, dk, dv) and not ctx.all_single    # values also transposed
         if self.own_kv and ctx.all_single:
             # one token a sequence: k and v go straight into the pages, then everything is read there
             ops.split_projection(proj, ctx.row_pos, self.proj_terms, nq, nkv, dk, dv, ng, q, None, None, gate,
@@ -174,21 +175,29 @@ class ScoredAttentionMixer(Mixer):
             k = ws.get("sattn_k" + tag, (n, nkv, dk), ctx.dtype)
             v = ws.get("sattn_v" + tag, (n, nkv, dv), ctx.dtype)
             ops.split_projection(proj, ctx.row_pos, self.proj_terms, nq, nkv, dk, dv, ng, q, k, v, gate)
+            if tiles:       # the matrix cores read values along the keys
+                vt = ws.get("sattn_vt" + tag, (nkv, dv, ctx.host["aligned_cols"]), ctx.dtype)
+                ops.v_tiles_rows(v, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, ctx.len_after)
             if run.kv_read_later:
-                ctx.host[f"kv_new_{run.index}"] = (k, v, None)
+                ctx.host[f"kv_new_{run.index}"] = (k, v, vt)
         else:
             ops.split_projection(proj, ctx.row_pos, self.proj_terms, nq, 0, dk, dv, ng, q, None, None, gate)
             if not ctx.all_single:
-                k, v, _ = ctx.host[f"kv_new_{run.kv_source}"]
+                k, v, vt = ctx.host[f"kv_new_{run.kv_source}"]
         if ctx.all_single:
             ops.attention_scored(q, None, None, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_after,
                                  self.terms, gate, att)
         else:
             ops.attention_scored(q, k, v, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_before,
-                                 self.terms, gate, att)
+                                 self.terms, gate, att, vt_new=vt)
             if self.own_kv:
                 def commit():
-                    ops.kv_commit_wide(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table, group.ring_pages, pages)
+                    if vt is not None and pages.dim() == 5:       # values a tile at a time, in whole lines
+                        ops.kv_commit_tiles(k, vt, ctx.row_seq, ctx.row_pos, ctx.tile_off, ctx.len_before,
+                                            ctx.len_after, table, group.ring_pages, pages)
+                    else:
+                        ops.kv_commit_wide(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table,
+                                           group.ring_pages, pages)
                 if run.kv_read_later:       # a later run still reads the old rows of the ring
                     ctx.host.setdefault("deferred", []).append(commit)
                 else:

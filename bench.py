@@ -40,6 +40,115 @@ SHAPES = {
 }
 
 
+# Layer sizes that resemble real models, for --only designs: both designs are built with these
+DESIGN_SIZES = {
+    "2b": dict(width=2048, heads=32, kv_heads=8, dim=64, ff=8192, window=1024, vocab=32000),
+    "7b": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, window=4096, vocab=32000),
+    "12b": dict(width=5120, heads=32, kv_heads=8, dim=128, ff=14336, window=None, vocab=131072),
+}
+
+
+def design_configs(z: dict, layers: int, share_from=None):
+    """config.json of a Sozetar and of a Mistral model with the layer sizes `z`.  `share_from`: the
+    Sozetar layers behind that index read its keys and values instead of making their own."""
+    def mixer(i):
+        m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
+             "scale": z["dim"] ** -0.5, "q_temp": {"coef": 0.3, "every": 128}}
+        if z["window"]:
+            m["mask"] = {"size": z["window"]}
+        if share_from is not None and i > share_from:
+            m["kv_from"] = share_from
+        return m
+    soz = {"architecture": "Sozetar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+           "layers": [{"type": "attention", "mixer": mixer(i), "mlp": {"kind": "dense", "ff": z["ff"]}}
+                      for i in range(layers)]}
+    mis = dict(architectures=["MistralForCausalLM"], num_hidden_layers=layers, hidden_size=z["width"],
+               num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+               intermediate_size=z["ff"], vocab_size=z["vocab"], rope_theta=10000.0, sliding_window=z["window"],
+               rms_norm_eps=1e-5)
+    return soz, mis
+
+
+def bench_designs(args) -> int:
+    """Prefill (one prompt of --prefill-tokens in one step) and decode (--batch sequences at --context
+    positions, one token a step through captured graphs) of the two designs at equal layer sizes,
+    random weights, bfloat16.  The bytes a decode step must read (every weight once, the live keys
+    and values) over its time is its share of the HBM roofline; a prefill's products and causal
+    attention over its time its share of the matrix cores' peak."""
+    import torch
+    from torchless_rs_amd import config_from_dict
+    from torchless_rs_amd.engine import Engine, SeqInput, model_from_tensors
+    from torchless_rs_amd.kernels.page import PAGE, round_up
+    from torchless_rs_amd.models import model_spec_for
+    from torchless_rs_amd.weights import random_tensors
+    dev = "cuda:0"
+    L = args.layers or 4
+    B, C, T = args.batch, min(args.context, 4096), args.prefill_tokens
+    gen = torch.Generator().manual_seed(11)
+    out = {"metric": "designs_side_by_side", "dtype": "bf16", "data": "synthetic", "layers": L, "batch": B,
+           "context": C, "prefill_tokens": T, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
+
+    def measure(cfgd, z, shared_layers=0):
+        cfg = config_from_dict(cfgd)
+        tensors = random_tensors(model_spec_for(cfg).weight_specs(), seed=5, std=0.02, dtype=torch.bfloat16, device=dev)
+        model = model_from_tensors(cfg, tensors, "bfloat16", dev)
+        del tensors
+        V = z["vocab"]
+        held = min(C, z["window"]) if z["window"] else C
+        eng = Engine(model, max_tokens=max(B * (round_up(held) + PAGE), round_up(T) + PAGE), max_slots=max(B, 1),
+                     freeze_gc=False)
+        # prefill
+        ids = torch.randint(0, V, (T,), generator=gen).tolist()
+        times = []
+        for i in range(2 + 3):
+            s = eng.alloc()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            eng.step([SeqInput(s, ids, [T - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            eng.free(s)
+        pre = min(times[2:])
+        # decode
+        slots = [eng.alloc() for _ in range(B)]
+        plen = max(1, C - args.steps - args.warmup - 1)
+        for s in slots:
+            p = torch.randint(0, V, (plen,), generator=gen).tolist()
+            for c0 in range(0, plen, 2048):
+                eng.step([SeqInput(s, p[c0:c0 + 2048], [])])
+        for _ in range(args.warmup + 2):                      # (the second step of a shape captures its graph)
+            eng.step([SeqInput(s, [7], [0]) for s in slots])
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(args.steps):
+            eng.step([SeqInput(s, [7], [0]) for s in slots])
+        torch.cuda.synchronize()
+        dec = (time.perf_counter() - t) / args.steps
+        for s in slots:
+            eng.free(s)
+        eng.close()
+        H, I, nq, nkv, d = z["width"], z["ff"], z["heads"], z["kv_heads"], z["dim"]
+        own = L - shared_layers
+        w_elems = L * (2 * nq * d * H + 3 * I * H) + own * 2 * nkv * d * H + V * H      # (biases, norms, gates: noise)
+        kv_bytes = B * held * 2 * nkv * d * 2 * L           # every layer reads its keys and values, shared or not
+        flops = 2 * T * (w_elems - V * H) + 2 * V * H + L * 4 * nq * d * sum(min(p + 1, z["window"] or T) for p in range(T))
+        return {"prefill_ms": round(pre * 1e3, 3), "prefill_tok_s": round(T / pre),
+                "prefill_frac_of_2.5_pflops": round(flops / pre / 2.5e15, 3),
+                "decode_ms": round(dec * 1e3, 3), "decode_tok_s": round(B / dec),
+                "decode_frac_of_8_tbs": round((2 * w_elems + kv_bytes) / dec / 8e12, 3)}
+
+    for name in [n for n in args.design_sizes.split(",") if n]:
+        z = DESIGN_SIZES[name]
+        soz, mis = design_configs(z, L)
+        row = {"sozetar": measure(soz, z), "mistral": measure(mis, z)}
+        if L > 2:
+            row["sozetar_sharing_keys"] = measure(design_configs(z, L, share_from=L // 2 - 1)[0], z, L - L // 2)
+        out["sizes"][name] = dict(z, **row)
+        print(f"[bench] {name}: {json.dumps(row)}", file=sys.stderr, flush=True)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,9 +168,13 @@ def main() -> int:
                     help="the baseline's configurations as it words them (unequal prompt lengths drawn from a seed, "
                          "256/128/128 new tokens, temperature 0.7 for the NeMo shape) run through the generation "
                          "loop, under 'workloads' (the default; --no-workloads skips them)")
-    ap.add_argument("--only", choices=["prefill", "decode", "pipes"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "pipes", "designs"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling); pipes: whether a "
-                         "SIMD's matrix and vector pipes overlap (ops.measure_pipes)")
+                         "SIMD's matrix and vector pipes overlap (ops.measure_pipes); designs: prefill and decode of "
+                         "the Sozetar design beside the Mistral design at equal layer sizes (--design-sizes, "
+                         "--layers, --batch, --context, --prefill-tokens apply)")
+    ap.add_argument("--design-sizes", default="2b,7b,12b",
+                    help="with --only designs: which layer sizes to run (of %s)" % ",".join(sorted(DESIGN_SIZES)))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not served")
@@ -72,6 +185,8 @@ def main() -> int:
         from torchless_rs_amd.kernels import ops as _o
         print(json.dumps({"pipes_ns_per_iteration": _o.measure_pipes("cuda:0")}), flush=True)
         return 0
+    if args.only == "designs":
+        return bench_designs(args)
     from torchless_rs_amd import SamplingConfig, config_from_dict
     from torchless_rs_amd.engine import Engine, SeqInput, model_from_tensors
     from torchless_rs_amd.engine.generate import BatchRun

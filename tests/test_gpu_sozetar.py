@@ -102,6 +102,34 @@ def test_gate_functions(activation):
     assert rel_err(out, want) < 1e-6
 
 
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+@pytest.mark.parametrize("K", [128, 192])                  # the ring of LDS stages takes multiples of 128, the other kernel the rest
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 64, 100, 128, 300])
+def test_the_gate_function_in_the_epilogue_of_the_product(activation, K, M):
+    """gate and up rows interleaved in blocks of 32: every kernel that a row count selects applies
+    act(gate) * up to its float sums itself; above the kernels' own rows the library's product is
+    followed by the same function on bfloat16 pairs."""
+    from torchless_rs_amd.kernels import ops
+    from torchless_rs_amd.parts.linear import interleave_pairs
+    g = torch.Generator().manual_seed(M + K)
+    I = 96
+    a = (torch.randn(M, K, generator=g) * 0.5).to(torch.bfloat16)
+    wg, wu = ((torch.randn(I, K, generator=g) * 0.2).to(torch.bfloat16) for _ in range(2))
+    w = dev(interleave_pairs(wg, wu))
+    out = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    if M > ops.own_rows(K):
+        gu = torch.empty(M, 2 * I, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_library(dev(a), w, gu)
+        ops.silu_mul_pairs(gu, out, activation)
+    elif M > 16:
+        ops.gemm_mid_bf16(dev(a), w, out, 1, silu_pair=True, pair_act=activation)
+    else:
+        ops.gemm_bf16(dev(a), w, out, silu_pair=True, pair_act=activation)
+    gate, up = a.double() @ wg.double().T, a.double() @ wu.double().T
+    act = plain.gelu_tanh(gate) if activation == "gelu_tanh" else gate / (1 + torch.exp(-gate))
+    assert rel_err(out, act * up) < (2e-2 if M > ops.own_rows(K) else 6e-3)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq, nkv, dk, dv, ng, temp, normed, biased", [
     (4, 2, 16, 32, 4, (0.5, 3), True, True),

@@ -203,6 +203,110 @@ split_projection_kernel(const float* __restrict__ proj, const int* __restrict__ 
   }
 }
 
+// The same, four channels at a time and three workgroups a row (blockIdx.y: q and the gate, k, v):
+// few rows, as in single-token steps, otherwise wait for one workgroup's chain of loads each.  All
+// of nq*dk, nkv*dk, nkv*dv and dk are multiples of 4 and the buffers 16-byte aligned.
+__device__ __forceinline__ float4 ld_f4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <typename T> __device__ __forceinline__ void st4(T* p, float4 a);
+template <> __device__ __forceinline__ void st4<float>(float* p, float4 a) { *reinterpret_cast<float4*>(p) = a; }
+template <> __device__ __forceinline__ void st4<bf16>(bf16* p, float4 a) {
+  bf16x4 o;
+  o[0] = (bf16)a.x; o[1] = (bf16)a.y; o[2] = (bf16)a.z; o[3] = (bf16)a.w;
+  *reinterpret_cast<bf16x4*>(p) = o;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+split_projection_vec_kernel(const float* __restrict__ proj, const int* __restrict__ row_pos, ProjectionTerms t,
+                            int nq, int nkv, int dk, int dv, int ng, T* __restrict__ q, T* __restrict__ k,
+                            T* __restrict__ v, float* __restrict__ gate, const int* __restrict__ table,
+                            int table_stride, int ring_pages, T* __restrict__ pages) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x, section = blockIdx.y;
+  const int Q = nq * dk, K = nkv * dk, V = nkv * dv;
+  const float* row = proj + (size_t)n * (Q + K + V + ng);
+  const int pos = row_pos[n];
+  // a piece of the row with its bias
+  auto piece = [&](int off, int c) {
+    float4 a = ld_f4(row + off + 4 * c);
+    if (t.bias) {
+      const float4 b = ld_f4(t.bias + off + 4 * c);
+      a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+    }
+    return a;
+  };
+  auto mean_square = [&](int off, int len) {
+    float ss = 0.f;
+#pragma unroll 4
+    for (int c = threadIdx.x; c < len / 4; c += 256) {
+      const float4 a = piece(off, c);
+      ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+    }
+    return block_sum<256>(ss, sh) / (float)len;
+  };
+  if (section == 0) {
+    float f = t.q_norm ? 1.0f / sqrtf(mean_square(0, Q) + t.eps) : 1.f;
+    float temp = 1.f;
+    if (t.temp_coef != 0.f) {
+      const float steps = (float)floor((double)(pos + 1) / (double)t.temp_every);
+      temp = 1.0f + t.temp_coef * logf(steps + 1.0f);
+    }
+#pragma unroll 4
+    for (int c = threadIdx.x; c < Q / 4; c += 256) {
+      float4 a = piece(0, c);
+      a.x *= f; a.y *= f; a.z *= f; a.w *= f;
+      if (t.q_norm) {
+        const float4 w = ld_f4(t.q_norm + 4 * c);
+        a.x *= w.x; a.y *= w.y; a.z *= w.z; a.w *= w.w;
+      }
+      a.x *= temp; a.y *= temp; a.z *= temp; a.w *= temp;
+      st4<T>(q + (size_t)n * Q + 4 * c, a);
+    }
+    for (int i = threadIdx.x; i < ng; i += 256) {
+      const float a = row[Q + K + V + i] + (t.bias ? t.bias[Q + K + V + i] : 0.f);
+      gate[(size_t)n * ng + i] = 1.0f / (1.0f + expf(-a));
+    }
+    return;
+  }
+  T* kd = nullptr;
+  T* vd = nullptr;
+  int r = 0;
+  if (pages) {
+    const int page = table[(size_t)n * table_stride + (pos / PAGE) % ring_pages];
+    kd = pages + (size_t)page * nkv * PAGE * (dk + dv);
+    vd = kd + (size_t)nkv * PAGE * dk;
+    r = pos % PAGE;
+  }
+  if (section == 1) {
+    const float f = t.k_norm ? 1.0f / sqrtf(mean_square(Q, K) + t.eps) : 1.f;
+#pragma unroll 4
+    for (int c = threadIdx.x; c < K / 4; c += 256) {
+      float4 a = piece(Q, c);
+      a.x *= f; a.y *= f; a.z *= f; a.w *= f;
+      if (t.k_norm) {
+        const float4 w = ld_f4(t.k_norm + 4 * c);
+        a.x *= w.x; a.y *= w.y; a.z *= w.z; a.w *= w.w;
+      }
+      const int i = 4 * c;
+      if (pages) st4<T>(kd + ((size_t)(i / dk) * PAGE + r) * dk + i % dk, a);
+      else st4<T>(k + (size_t)n * K + i, a);
+    }
+    return;
+  }
+#pragma unroll 4
+  for (int c = threadIdx.x; c < V / 4; c += 256) {
+    const float4 a = piece(Q + K, c);
+    const int i = 4 * c;
+    if (pages) {
+      const float e[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) vd[((size_t)((i + u) / dv) * dv + (i + u) % dv) * PAGE + r] = from_f32<T>(e[u]);
+    } else {
+      st4<T>(v + (size_t)n * V + i, a);
+    }
+  }
+}
+
 // Rows of keys [n, nkv, dk] and values [n, nkv, dv] into the pages of their positions.  A row
 // that the same step overwrites in a ring (older than the ring is long) is skipped.
 template <typename T>
@@ -277,6 +381,21 @@ int tl_split_projection(const float* proj, const int* row_pos, const float* bias
   TL_REQUIRE(temp_coef == 0.f || temp_every > 0.f, "split_projection: the factor on q needs a positive step");
   if (n == 0) return 0;
   const ProjectionTerms t{bias, q_norm, k_norm, eps, temp_coef, temp_every};
+  const int Q = nq * dk, K = nkv * dk, V = nkv * dv;
+  auto al = [](const void* p) { return (uintptr_t)p % 16 == 0; };
+  const bool vec = Q % 4 == 0 && K % 4 == 0 && V % 4 == 0 && dk % 4 == 0 && ng % 4 == 0 && al(proj) && al(bias) &&
+                   al(q_norm) && al(k_norm) && al(q) && al(k) && al(v) && al(pages);
+  if (vec && (dt == DT_F32 || dt == DT_BF16)) {
+    const dim3 grid(n, nkv > 0 ? 3 : 1);
+    if (dt == DT_F32)
+      split_projection_vec_kernel<float><<<grid, 256, 0, st>>>(proj, row_pos, t, nq, nkv, dk, dv, ng, (float*)q, (float*)k,
+                                                               (float*)v, gate, table, table_stride, ring_pages, (float*)pages);
+    else
+      split_projection_vec_kernel<bf16><<<grid, 256, 0, st>>>(proj, row_pos, t, nq, nkv, dk, dv, ng, (bf16*)q, (bf16*)k,
+                                                              (bf16*)v, gate, table, table_stride, ring_pages, (bf16*)pages);
+    TL_LAUNCH_CHECK("split_projection");
+    return 0;
+  }
   if (dt == DT_F32)
     split_projection_kernel<float><<<n, 256, 0, st>>>(proj, row_pos, t, nq, nkv, dk, dv, ng, (float*)q, (float*)k,
                                                      (float*)v, gate, table, table_stride, ring_pages, (float*)pages);

@@ -425,6 +425,16 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
   }
 }
 
+// ---- the function of a gated feed-forward's gate ---------------------------------
+// 0: silu(g) = g / (1 + exp(-g)); 1: the tanh form of gelu,
+// 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+constexpr int ACT_SILU = 0;
+constexpr int ACT_GELU_TANH = 1;
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.0f + expf(-g));
+}
+
 // ---- h = silu(gate) * up, silu(g) = g / (1 + exp(-g)) ------------------------
 // src/kernels/mod.rs:546-548, src/model/modules/mlp.rs:33-39.
 template <typename TO>
@@ -440,7 +450,7 @@ __global__ void silu_mul_kernel(const float* __restrict__ gu, int I, TO* __restr
 // gu[n, 2I] in bfloat16 with columns in groups of 64 (32 of gate, then the 32 of up
 // that belong to them); out[n, I] = silu(gate) * up.  A thread takes 8 pairs.
 __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chunks, int I,
-                                      bf16* __restrict__ out) {
+                                      bf16* __restrict__ out, int act = ACT_SILU) {
   const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= chunks) return;
   const int per_row = I / 8;
@@ -453,7 +463,7 @@ __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chu
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const float gv = (float)g[t];
-    o[t] = (bf16)((gv / (1.0f + expf(-gv))) * (float)u[t]);
+    o[t] = (bf16)(gate_act(gv, act) * (float)u[t]);
   }
   *reinterpret_cast<bf16x8*>(out + n * I + group * 32 + part * 8) = o;
 }
@@ -553,16 +563,6 @@ layernorm_reg_kernel(const float* __restrict__ z, const float* __restrict__ bias
 __global__ void cast_rows_kernel(const float* __restrict__ x, size_t total, bf16* __restrict__ out) {
   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < total) out[i] = (bf16)x[i];
-}
-
-// ---- the function of a gated feed-forward's gate ---------------------------------
-// 0: silu(g) = g / (1 + exp(-g)); 1: the tanh form of gelu,
-// 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
-constexpr int ACT_SILU = 0;
-constexpr int ACT_GELU_TANH = 1;
-__device__ __forceinline__ float gate_act(float g, int act) {
-  if (act == ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-  return g / (1.0f + expf(-g));
 }
 
 // h = act(gate) * up from gu[n, 2I] = [gate | up]
@@ -921,6 +921,19 @@ int tl_act_mul(const float* gu, int n, int I, int act, void* out, int out_dt, hi
   else
     TL_REQUIRE(false, "act_mul: unknown dtype code %d", out_dt);
   TL_LAUNCH_CHECK("act_mul");
+  return 0;
+}
+
+// tl_silu_mul_pairs with the gate's function chosen (codes as tl_act_mul)
+int tl_act_mul_pairs(const void* gu, int n, int I, int act, void* out, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && I > 0 && I % 32 == 0, "act_mul_pairs: bad sizes n=%d I=%d (I in steps of 32)", n, I);
+  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH, "act_mul_pairs: no function of code %d", act);
+  TL_REQUIRE((uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0, "act_mul_pairs: buffers must be 16-byte aligned");
+  if (n == 0) return 0;
+  const long long chunks = (long long)n * (I / 8);
+  TL_REQUIRE((chunks + 255) / 256 < 2147483647LL, "act_mul_pairs: too many elements");
+  silu_mul_pairs_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const bf16*)gu, chunks, I, (bf16*)out, act);
+  TL_LAUNCH_CHECK("act_mul_pairs");
   return 0;
 }
 

@@ -48,6 +48,16 @@ constexpr int EPI_STORE = 0;        // C = product (float)
 constexpr int EPI_ACCUMULATE = 1;   // C += product (float; the residual stream)
 constexpr int EPI_SILU_PAIR = 2;    // W's rows come in groups of 64 (32 gate rows, their 32 up rows):
                                     // C is bfloat16 [M, N/2] = silu(gate) * up
+constexpr int EPI_GELU_PAIR = 3;    // the same pairs with the tanh form of gelu on the gate:
+                                    // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+__host__ __device__ __forceinline__ bool is_pair(int epilogue) {
+  return epilogue == EPI_SILU_PAIR || epilogue == EPI_GELU_PAIR;
+}
+// the gate's function in a paired epilogue, on the float sums
+__device__ __forceinline__ float pair_act(float g, int epilogue) {
+  if (epilogue == EPI_GELU_PAIR) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.0f + expf(-g));
+}
 
 // An RMSNorm cut in two around a product of at most 16 rows, so that the norm needs no
 // kernel of its own.  The product that completes the residual stream (accumulate epilogue)
@@ -246,7 +256,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     for (int w = 0; w < SK_WAVES; ++w) v += red[w][idx];
     return scaled ? v * rs[m % 16] : v;
   };
-  if (epilogue == EPI_SILU_PAIR) {
+  if (is_pair(epilogue)) {
     // rows come in groups of 64: 32 gate rows, then the 32 up rows that belong to them
     if constexpr (NB % 64 == 0) {
       bf16* H = reinterpret_cast<bf16*>(C);
@@ -257,7 +267,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
         const int n = (n0 / 2) + jl;
         if (n < NH && m < M) {
           const float g = total(grp * 64 + j, m), u = total(grp * 64 + 32 + j, m);
-          H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * u);
+          H[(size_t)m * NH + n] = (bf16)(pair_act(g, epilogue) * u);
         }
       }
     }
@@ -421,14 +431,14 @@ gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
     for (int w = 0; w < 4; ++w) v += red[w * (NRB * 256) + idx];
     return scaled ? v * rs[m] : v;
   };
-  if (epilogue == EPI_SILU_PAIR) {                     // the 64 rows are 32 gate rows and their 32 up rows
+  if (is_pair(epilogue)) {                     // the 64 rows are 32 gate rows and their 32 up rows
     bf16* H = reinterpret_cast<bf16*>(C);
     const int NH = N / 2;
     for (int e = threadIdx.x; e < 32 * 16; e += 256) {
       const int j = e % 32, m = e / 32;
       if (m < M) {
         const float g = total(j, m), u = total(32 + j, m);
-        H[(size_t)m * NH + n0 / 2 + j] = (bf16)((g / (1.0f + expf(-g))) * u);
+        H[(size_t)m * NH + n0 / 2 + j] = (bf16)(pair_act(g, epilogue) * u);
       }
     }
     return;
@@ -696,7 +706,7 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
     }
   }
   // acc[u][r] = D[m = 16 u + 4 kg + r][n = n0 + li]
-  if (epilogue == EPI_SILU_PAIR) {
+  if (is_pair(epilogue)) {
     // the workgroup's 64 rows are one group: waves 0,1 hold gate rows, waves 2,3 their up rows
     __syncthreads();
     float* ex = reinterpret_cast<float*>(&As[0]);           // [2 waves][MT][4][64] floats: 2 KB a row tile
@@ -718,7 +728,7 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
           const int m = 16 * u + 4 * kg + r;
           if (m < M && n < NH) {
             const float g = acc[u][r], up = ex[((wave * MT + u) * 4 + r) * 64 + lane];
-            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * up);
+            H[(size_t)m * NH + n] = (bf16)(pair_act(g, epilogue) * up);
           }
         }
     }
@@ -869,7 +879,7 @@ gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
         acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(areg[u][j], wreg[j], acc[u], 0, 0, 0);
   }
   // acc[u][r] = D[m = 16 u + 4 kg + r][n = n0 + li]
-  if (epilogue == EPI_SILU_PAIR) {
+  if (is_pair(epilogue)) {
     // the workgroup's channels are groups of 64: of a group's four waves, the first two hold gate
     // rows, the other two their up rows
     __builtin_amdgcn_s_barrier();                           // the ring is free
@@ -893,7 +903,7 @@ gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
           const int m = 16 * u + 4 * kg + r;
           if (m < M && n < NH) {
             const float g = acc[u][r], up = ex[(((grp * 2 + wq) * MT + u) * 4 + r) * 64 + lane];
-            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * up);
+            H[(size_t)m * NH + n] = (bf16)(pair_act(g, epilogue) * up);
           }
         }
     }
@@ -962,17 +972,17 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, int wt
   TL_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0),
              "gemm_bf16: operands must be 16-byte aligned");
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16: unknown epilogue %d", epilogue);
-  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_bf16: unknown epilogue %d", epilogue);
+  TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   if (M == 0) return 0;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   float* c = (float*)C;
-  const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;     // many rows: 64 a workgroup
+  const bool wide = N >= 16384 || is_pair(epilogue);     // many rows: 64 a workgroup
   if (M <= 16) {
     if (wide && rows_fit(M, N, K)) return launch_rows(a, w, c, M, N, K, epilogue, st);
-    if (wide && (M > 4 || epilogue == EPI_SILU_PAIR)) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
+    if (wide && (M > 4 || is_pair(epilogue))) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
     return launch_shares(a, w, (const bf16*)Wt, wt_height, c, M, N, K, epilogue, st, NormSplit{}, balanced_share(N));
   }
   if (M <= 32) {
@@ -992,7 +1002,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, int wt
 extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M, int N, int K,
                                     int epilogue, int variant, hipStream_t st) {
   TL_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
-  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
+  TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
@@ -1003,14 +1013,14 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
     return launch_rows(a, w, c, M, N, K, epilogue, st);
   }
   if (variant > 1000 && variant <= 1032) {
-    TL_REQUIRE(M <= 16 && epilogue != EPI_SILU_PAIR, "gemm_skinny: variant %d takes at most 16 rows and no pairs", variant);
+    TL_REQUIRE(M <= 16 && !is_pair(epilogue), "gemm_skinny: variant %d takes at most 16 rows and no pairs", variant);
     const int R = variant - 1000;
     if (R <= 16) return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);
     return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);
   }
   const int mt = (variant / 10) % 10;
   TL_REQUIRE(M <= 16 * mt, "gemm_skinny: variant %d takes at most %d rows, not %d", variant, 16 * mt, M);
-  TL_REQUIRE(epilogue != EPI_SILU_PAIR || variant / 100 == 4, "gemm_skinny: the paired epilogue needs 64 rows "
+  TL_REQUIRE(!is_pair(epilogue) || variant / 100 == 4, "gemm_skinny: the paired epilogue needs 64 rows "
              "a workgroup (variant 4xx)");
   switch (variant) {
     case 112: return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st);
@@ -1041,9 +1051,9 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
   TL_REQUIRE(n_split >= 1 && n_split <= (K + MID_KS - 1) / MID_KS && n_split <= 65535,
              "gemm_mid: %d splits do not fit K=%d (one step of %d at least each)", n_split, K, MID_KS);
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 2 && (n_split == 1 || epilogue == EPI_STORE),
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 3 && (n_split == 1 || epilogue == EPI_STORE),
              "gemm_mid: epilogue %d cannot go with %d splits", epilogue, n_split);
-  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_mid: the paired epilogue needs N=%d to be a "
+  TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_mid: the paired epilogue needs N=%d to be a "
              "multiple of 64", N);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
@@ -1069,9 +1079,9 @@ extern "C" int tl_gemm_ring_bf16(const void* A, const void* W, void* C, int M, i
   TL_REQUIRE(kc == 64 || kc == 128, "gemm_ring: a stage of %d k (64 or 128)", kc);
   TL_REQUIRE(n_split >= 1 && n_split <= K / kc && n_split <= 65535,
              "gemm_ring: %d splits do not fit K=%d (one stage of %d at least each)", n_split, K, kc);
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 2 && (n_split == 1 || epilogue == EPI_STORE),
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 3 && (n_split == 1 || epilogue == EPI_STORE),
              "gemm_ring: epilogue %d cannot go with %d splits", epilogue, n_split);
-  TL_REQUIRE(epilogue != EPI_SILU_PAIR || (N % 64 == 0 && waves % 4 == 0), "gemm_ring: the paired epilogue needs N=%d "
+  TL_REQUIRE(!is_pair(epilogue) || (N % 64 == 0 && waves % 4 == 0), "gemm_ring: the paired epilogue needs N=%d "
              "to be a multiple of 64 and whole groups of four waves (%d)", N, waves);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
@@ -1157,16 +1167,16 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, i
   TL_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16_norm: bad sizes M=%d N=%d K=%d (at most "
              "16 rows, K a multiple of 8)", M, N, K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_bf16_norm: operands must be 16-byte aligned");
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16_norm: unknown epilogue %d", epilogue);
-  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16_norm: the paired epilogue needs N=%d to be "
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_bf16_norm: unknown epilogue %d", epilogue);
+  TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16_norm: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   TL_REQUIRE(ssq_in == nullptr || n_part > 0, "gemm_bf16_norm: %d partial sums of squares", n_part);
   const bool writer = norm_w != nullptr;
   TL_REQUIRE(!writer || (epilogue == EPI_ACCUMULATE && xt != nullptr && ssq_out != nullptr),
              "gemm_bf16_norm: the next norm's half goes with the accumulate epilogue, xt and ssq_out");
-  const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;
+  const bool wide = N >= 16384 || is_pair(epilogue);
   const bool rows = wide && !writer && rows_fit(M, N, K);        // many channels, K in chunks of 512: whole rows, 1 KB a load
-  const bool four = wide && (M > 4 || epilogue == EPI_SILU_PAIR);
+  const bool four = wide && (M > 4 || is_pair(epilogue));
   const int share = four ? 64 : balanced_share(N);
   const int groups = (N + share - 1) / share;
   if (n_groups) *n_groups = groups;

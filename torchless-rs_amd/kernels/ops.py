@@ -295,13 +295,19 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().tl_silu_mul(_p(gu), n, I2 // 2, _p(out), _code(out.dtype), _stream()))
 
 
-def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor) -> None:
+def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
     """The same on bfloat16 gu whose columns come in groups of 64: 32 of gate,
-    then the 32 of up that belong to them (`interleave_pairs`)."""
+    then the 32 of up that belong to them (`interleave_pairs`); `activation`: the gate's
+    function (`ACTIVATIONS`)."""
     n, I2 = gu.shape
     _req(gu, "silu_mul_pairs.gu", torch.bfloat16)
     _req(out, "silu_mul_pairs.out", torch.bfloat16, (n, I2 // 2))
-    _check(lib().tl_silu_mul_pairs(_p(gu), n, I2 // 2, _p(out), _stream()))
+    if activation == "silu":
+        _check(lib().tl_silu_mul_pairs(_p(gu), n, I2 // 2, _p(out), _stream()))
+        return
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"silu_mul_pairs: no function {activation!r}; there are {sorted(ACTIVATIONS)}")
+    _check(lib().tl_act_mul_pairs(_p(gu), n, I2 // 2, ACTIVATIONS[activation], _p(out), _stream()))
 
 
 def layernorm(z: torch.Tensor, w: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
@@ -547,7 +553,14 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, s
                            _p(counters), _p(probs), _p(out), _stream()))
 
 
-EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR = 0, 1, 2
+EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR, EPI_GELU_PAIR = 0, 1, 2, 3
+
+
+def _pair_epilogue(pair_act: str) -> int:
+    """The code of the paired epilogue act(gate) * up for the gate's function `pair_act`."""
+    if pair_act not in ACTIVATIONS:
+        raise KernelError(f"paired epilogue: no function {pair_act!r}; there are {sorted(ACTIVATIONS)}")
+    return EPI_GELU_PAIR if pair_act == "gelu_tanh" else EPI_SILU_PAIR
 
 
 def tiles_fit(N: int, K: int) -> bool:
@@ -614,7 +627,7 @@ def _req_tiles(tiles: Optional[torch.Tensor], N: int, K: int, height: Optional[i
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
               variant: Optional[int] = None, silu_pair: bool = False,
-              tiles: Optional[torch.Tensor] = None) -> None:
+              tiles: Optional[torch.Tensor] = None, pair_act: str = "silu") -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T on the matrix cores: bfloat16 operands,
     float32 accumulation.  K must be a multiple of 8.  With `silu_pair`, w's
     rows come in groups of 64 (32 gate rows and the 32 up rows that belong to
@@ -630,7 +643,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         if accumulate or N % 64:
             raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
         _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
-        epi = EPI_SILU_PAIR
+        epi = _pair_epilogue(pair_act)
     else:
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE
@@ -657,7 +670,7 @@ def norm_split_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
                    silu_pair: bool = False, factor: Optional[RowFactor] = None,
                    norm_weight: Optional[torch.Tensor] = None, xt: Optional[torch.Tensor] = None,
-                   ssq_out: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None) -> int:
+                   ssq_out: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None, pair_act: str = "silu") -> int:
     """`gemm_bf16` for at most 16 rows with the halves of an RMSNorm around it.
     `factor`: every row of the result is multiplied by its rsqrt(mean(x^2) + eps).
     `norm_weight`, `xt`, `ssq_out` (with `accumulate`): out += product, xt =
@@ -672,7 +685,7 @@ def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumula
         if accumulate or N % 64:
             raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
         _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
-        epi = EPI_SILU_PAIR
+        epi = _pair_epilogue(pair_act)
     else:
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE
@@ -745,7 +758,7 @@ def mid_splits(M: int, N: int, K: int, units: int) -> int:
 
 
 def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: int = 1,
-                  accumulate: bool = False, silu_pair: bool = False) -> None:
+                  accumulate: bool = False, silu_pair: bool = False, pair_act: str = "silu") -> None:
     """The product for 17..MID_ROWS rows (the ring kernel where K is a multiple of RING_K, else
     gemm_mid).  n_split == 1: out as in `gemm_bf16`.  n_split > 1: out is float32 [n_split, M, N]
     and receives partial sums that the next kernel adds up (`add_rmsnorm`, `add_partials`,
@@ -761,7 +774,7 @@ def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: 
         epi = EPI_STORE
     elif silu_pair:
         _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
-        epi = EPI_SILU_PAIR
+        epi = _pair_epilogue(pair_act)
     else:
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE
@@ -769,7 +782,7 @@ def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: 
 
 
 def gemm_ring_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: int = 1, accumulate: bool = False,
-                   silu_pair: bool = False, waves: int = 4, kc: int = 128) -> None:
+                   silu_pair: bool = False, waves: int = 4, kc: int = 128, pair_act: str = "silu") -> None:
     """`gemm_mid_bf16` through the kernel that brings both operands into a ring of stages in LDS
     (K a multiple of 128); `waves`: 4, 7 or 8 waves a workgroup with 16 channels each; `kc`: the k
     of a stage, 64 or 128."""
@@ -784,7 +797,7 @@ def gemm_ring_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split:
         epi = EPI_STORE
     elif silu_pair:
         _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
-        epi = EPI_SILU_PAIR
+        epi = _pair_epilogue(pair_act)
     else:
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE

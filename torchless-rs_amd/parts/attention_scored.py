@@ -130,8 +130,8 @@ class ScoredAttentionMixer(Mixer):
         ws = [t("q")] + ([t("k"), t("v")] if self.own_kv else []) + ([t("gate")] if self.head_gate else [])
         if len({w.dtype for w in ws}) > 1:
             ws = [w.to(torch.float32) for w in ws]
-        self.proj = Linear(torch.cat(ws, dim=0))
-        self.o = Linear(t("o"))
+        self.proj = Linear(torch.cat(ws, dim=0), tiled=True)      # single-token steps stream both from tiled copies
+        self.o = Linear(t("o"), tiled=True)
         dev = ws[0].device
         bias = None
         if self.bias:

@@ -62,7 +62,7 @@ class SwiGLU(FeedForward):
         # bfloat16 on the matrix cores: gate and up rows interleaved so that the product's
         # epilogue applies silu(gate) * up itself and writes bfloat16
         self.paired = (compute_dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and self.I % 32 == 0
-                       and self.H % 8 == 0 and self.activation == "silu")
+                       and self.H % 8 == 0)
         self.gate_up = Linear(interleave_pairs(g, u) if self.paired else torch.cat([g, u], dim=0))
         self.down = Linear(tensors[p + nm["down"]], tiled=True)
 
@@ -78,16 +78,16 @@ class SwiGLU(FeedForward):
         h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
         factor = take_row_factor(ctx, usable=self.paired and ops.norm_split_ok(y, self.gate_up.weight))
         if factor is not None:
-            ops.gemm_bf16_norm(y, self.gate_up.weight, h, silu_pair=True, factor=factor)
+            ops.gemm_bf16_norm(y, self.gate_up.weight, h, silu_pair=True, factor=factor, pair_act=self.activation)
         elif self.paired and self.gate_up.mid(y):
-            ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True)
+            ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True, pair_act=self.activation)
         elif self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
             if n > ops.LIBRARY_ROWS:
                 gu = ctx.workspace.get("ffn_gu16", (n, 2 * self.I), torch.bfloat16)
                 ops.gemm_library(y, self.gate_up.weight, gu)
-                ops.silu_mul_pairs(gu, h)
+                ops.silu_mul_pairs(gu, h, self.activation)
             else:
-                ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True)
+                ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True, pair_act=self.activation)
         else:
             gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
             self.gate_up(y, gu)

@@ -46,8 +46,14 @@ CORES = {"architecture": "Sozetar", "vocab": 256, "width": 128, "norm": {"eps": 
     layer(att(4, 1, 32, 64, 0.18, temp=(0.3, 40)), ff=64),
     layer(att(4, 1, 32, 64, 0.18, window=40, kv_from=2)),
 ]}
-CONFIGS = {"mixed": MIXED, "wide": WIDE, "ones": ONES, "cores": CORES}
-LENGTHS = {"mixed": [1, 7, 23, 70], "wide": [3, 66, 150, 290], "ones": [2, 65, 130, 200], "cores": [5, 64, 129, 330]}
+# sizes that no kernel's fast way takes: a width that is no multiple of 8, heads of 12 and 20, 5 heads, an odd vocabulary
+ODD = {"architecture": "Sozetar", "vocab": 131, "width": 100, "norm": {"eps": 1e-5}, "layers": [
+    layer(att(5, 5, 12, 20, 0.29, window=33, temp=(0.25, 10)), ff=50),
+    layer(att(5, 5, 12, 20, 0.29, kv_from=0, temp=(0.6, 2.5)), ff=36),
+]}
+CONFIGS = {"mixed": MIXED, "wide": WIDE, "ones": ONES, "cores": CORES, "odd": ODD}
+LENGTHS = {"mixed": [1, 7, 23, 70], "wide": [3, 66, 150, 290], "ones": [2, 65, 130, 200], "cores": [5, 64, 129, 330],
+           "odd": [4, 33, 67, 140]}
 NAMES = list(CONFIGS)
 
 
@@ -256,7 +262,8 @@ ATT_TOL = {"float32": 2e-5, "bfloat16": 1.2e-2}
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("what", ["nothing", "slopes", "sink", "window", "gate", "all"])
 @pytest.mark.parametrize("nq, nkv, dk, dv", [(4, 2, 16, 32), (6, 3, 40, 24), (8, 2, 64, 64), (4, 1, 32, 64), (1, 1, 8, 8),
-                                             (6, 1, 48, 48), (20, 1, 128, 128), (3, 3, 80, 80)])
+                                             (6, 1, 48, 48), (20, 1, 128, 128), (3, 3, 80, 80), (2, 1, 256, 256),
+                                             (34, 2, 96, 96)])
 def test_attention_terms_one_by_one(dtype, what, nq, nkv, dk, dv):
     slopes = plain.head_slopes(nq) if what in ("slopes", "all") else None
     sinks = torch.linspace(-1, 2, nq, dtype=torch.float64) if what in ("sink", "all") else None
@@ -597,7 +604,7 @@ def test_the_command_line_and_the_trace_replay(zoo, tmp_path):
              {"step": 2, "entries": [{"id": "a", "tokens": [p[21]], "want": [0]}], "end": ["a"]}]
     out = tmp_path / "logits"
     r = subprocess.run([sys.executable, os.path.join(REPO, "bin", "trace_run"), "--model", z["dir"], "--dtype", "float32",
-                        "--out", str(out), "--max-tokens", "256"], input="\n".join(json.dumps(s) for s in steps) + "\n",
+                        "--out", str(out), "--max-tokens", "23"], input="\n".join(json.dumps(s) for s in steps) + "\n",
                        capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     assert [l for l in r.stdout.split("\n") if l.startswith("done")] == ["done 0", "done 1", "done 2"]

@@ -35,7 +35,8 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder that receives <step>.f32")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each rounded up to whole pages of the cache, 64)")
+                    help="most tokens live requests hold at any time (the rounding of each request to whole pages "
+                         "of the cache is added here)")
     args = ap.parse_args(argv)
 
     print("[trace_run] loading torch and the kernels", file=sys.stderr, flush=True)
@@ -44,7 +45,9 @@ def main(argv=None) -> int:
     os.makedirs(args.out, exist_ok=True)
     model = load_model(args.model, args.dtype, "cuda:0")
     from ..kernels.page import PAGE
-    engine = Engine(model, max_tokens=max(args.max_tokens, PAGE))
+    # every live request may leave most of a page unused: room for that beside the tokens themselves
+    most_requests = min(max(args.max_tokens, 1), 256)
+    engine = Engine(model, max_tokens=max(args.max_tokens, PAGE) + PAGE * most_requests)
     print("[trace_run] ready", file=sys.stderr, flush=True)
 
     slot_of: Dict[str, int] = {}

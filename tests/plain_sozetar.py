@@ -65,14 +65,15 @@ def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
 
 
 def attend(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, slopes: Optional[torch.Tensor],
-           sinks: Optional[torch.Tensor], window: Optional[int]) -> torch.Tensor:
-    """q [n, H, dk], k [n, G, dk], v [n, G, dv] -> [n, H, dv].  Row by row and key by key."""
+           sinks: Optional[torch.Tensor], window: Optional[int], first_row: int = 0) -> torch.Tensor:
+    """q [n, H, dk], k [n, G, dk], v [n, G, dv] -> [n, H, dv].  Row by row and key by key.  Rows before
+    `first_row` are left zero (a caller that asks for the last rows only)."""
     n, H, _ = q.shape
     G = k.shape[1]
     out = torch.zeros(n, H, v.shape[2], dtype=F)
     for h in range(H):
         g = h // (H // G)
-        for p in range(n):
+        for p in range(first_row, n):
             lo = 0 if window is None else max(0, p - window + 1)
             s = (k[lo:p + 1, g] @ q[p, h]) * scale
             if slopes is not None:

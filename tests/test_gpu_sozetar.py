@@ -250,7 +250,7 @@ def attention_case(dtype, nq, nkv, dk, dv, cached, new, window, slopes, sinks, g
         ops.attention_scored(q, k_new, v_new, pages, nkv, dv, table, ring, ctx, ctx.len_before, terms,
                              dev(gate) if gated else None, out, vt_new=vt)
     want = torch.cat([plain.attend(seqs[b][0].double(), seqs[b][1].double(), seqs[b][2].double(), scale,
-                                   slopes, sinks, window)[cached[b]:] for b in range(B)])
+                                   slopes, sinks, window, first_row=cached[b])[cached[b]:] for b in range(B)])
     if gated:
         want = want * gate.double()[:, :, None]
     return out, want
@@ -347,6 +347,18 @@ def test_a_far_key_among_hundreds_and_the_sink_alone(dtype):
     got, want = attention_case(dtype, nq, nkv, dk, dv, [10], [20], None, None, torch.full((nq,), 40.0, dtype=torch.float64),
                                False, 12)
     assert got.float().abs().max() < 1e-6 and want.abs().max() < 1e-6
+
+
+@pytest.mark.parametrize("window", [None, 1000])
+@pytest.mark.parametrize("nq, nkv, d", [(8, 2, 64), (4, 1, 128), (6, 3, 48), (2, 2, 256)])
+def test_single_tokens_over_long_contexts_in_several_splits(nq, nkv, d, window):
+    """Sequences of very unequal lengths, one token each: the keys of the long ones are cut over several
+    workgroups whose sums are merged; the sink must count once, in whichever split, and the gate once."""
+    sinks = torch.linspace(-2, 3, nq, dtype=torch.float64)
+    for cached in ([2500, 70, 1300], [4000], [63, 64, 65, 1]):
+        got, want = attention_case("bfloat16", nq, nkv, d, d, cached, [1] * len(cached), window,
+                                   plain.head_slopes(nq) * 0.05, sinks, True, seed=d)
+        assert rel_err(got, want) < ATT_TOL["bfloat16"], (cached,)
 
 
 # ---------------------------------------------------------------------------------------------

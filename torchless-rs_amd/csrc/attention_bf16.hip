@@ -734,12 +734,13 @@ template <int N> __device__ __forceinline__ void wait_page_loads_but() {     // 
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int D, int NS>
+template <int D, int NS, bool TERMS = false>
 __global__ void __launch_bounds__(DC_WAVES * 64)
 attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                         const int* __restrict__ table, int table_stride, int ring_pages,
                         const int* __restrict__ row_pos, int nq, int nkv, int window, float scale,
-                        int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out) {
+                        int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out,
+                        MoreTerms terms) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char dr_smem[];
   constexpr int KB = D / 32, VB = D / 16;
   constexpr int K_BYTES = PAGE * D * 2, STAGE = 2 * K_BYTES;   // keys, then values, as many bytes each
@@ -808,6 +809,9 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
 #pragma unroll
   for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
+  float slope = 0.f;
+  if constexpr (TERMS)
+    if (terms.slopes != nullptr) slope = terms.slopes[h];
 
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
@@ -840,7 +844,8 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int j = j0 + 4 * kg + r;
-      sv[r] = (j <= p && j >= lo) ? s[r] * scale : -INFINITY;
+      if constexpr (TERMS) sv[r] = (j <= p && j >= lo) ? s[r] * scale - slope * (float)(p - j) : -INFINITY;
+      else sv[r] = (j <= p && j >= lo) ? s[r] * scale : -INFINITY;
       tmax = fmaxf(tmax, sv[r]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
@@ -848,12 +853,13 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
     const float m_new = fmaxf(m, tmax);               // finite: one of the 16 keys is visible
     const float alpha = __expf(m - m_new);
     float psum = 0.f;
-    bf16x4 pb;
+    bf16x4 pb, pb_lo;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float pv = __expf(sv[r] - m_new);
       psum += pv;
       pb[r] = (bf16)pv;
+      if constexpr (TERMS) pb_lo[r] = (bf16)(pv - (float)pb[r]);
     }
     psum += __shfl_xor(psum, 16, WAVE);
     psum += __shfl_xor(psum, 32, WAVE);
@@ -878,6 +884,11 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
     const s16x4 pbits = __builtin_bit_cast(s16x4, pb);
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb) o[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[vb], pbits, o[vb], 0, 0, 0);
+    if constexpr (TERMS) {                            // what the rounding of the weights left over
+      const s16x4 lbits = __builtin_bit_cast(s16x4, pb_lo);
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) o[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[vb], lbits, o[vb], 0, 0, 0);
+    }
   }
   // o[vb][r] = O[dv = 16 vb + 4 kg + r][head li]; m, l are per head li (equal in the 4 kg lanes).
   // Merge the waves in the ring's memory: common maximum, then every wave's scaled share.
@@ -915,8 +926,21 @@ attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pag
 #pragma unroll
     for (int w = 1; w < DC_WAVES; ++w) osum += red_o[w * (VB * 4 * 64) + idx];
     const size_t bh = (size_t)b * nq + kvh * g + hg * 16 + hd;
+    if constexpr (TERMS) {
+      if (terms.sinks != nullptr && split == 0) {     // the sink counts once: with the first split
+        const float sk = terms.sinks[kvh * g + hg * 16 + hd];
+        const float ms = fmaxf(mh, sk);
+        const float fs = (mh == -INFINITY) ? 0.f : __expf(mh - ms);
+        ll = ll * fs + __expf(sk - ms);
+        osum *= fs;
+        mh = ms;
+      }
+    }
     if (n_splits == 1) {
-      out[bh * D + dv] = (bf16)(osum / ll);
+      float res = osum / ll;
+      if constexpr (TERMS)
+        if (terms.gate != nullptr) res *= terms.gate[bh];
+      out[bh * D + dv] = (bf16)res;
       continue;
     }
     float* dst = part + (bh * n_splits + split) * (D + 2);
@@ -1059,7 +1083,32 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
                          float scale, int n_splits, float* part, bf16* out, hipStream_t st, const MoreTerms* terms) {
   const int g = nq / nkv, head_groups = (g + 15) / 16;
   dim3 grid(B * nkv * head_groups, n_splits);
-  if (terms != nullptr) {         // more terms on the scores: the kernel that reads the pages into registers
+  if constexpr (DPAD == 64 || DPAD == 128 || DPAD == 256) {
+    if (terms != nullptr && d == DPAD && decode_through_lds && table_stride <= DR_MAX_PAGES) {
+      constexpr int NS = DPAD == 64 ? 4 : 2;
+      constexpr int LDS = NS * PAGE * DPAD * 4 + DR_MAX_PAGES * 4;
+      static bool raised_terms = false;
+      if (!raised_terms) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_decode_ring_kernel<DPAD, NS, true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (e != hipSuccess) {
+          set_error("attn_decode: cannot have %d bytes of LDS: %s", LDS, hipGetErrorString(e));
+          return 2;
+        }
+        raised_terms = true;
+      }
+      attn_decode_ring_kernel<DPAD, NS, true><<<grid, DC_WAVES * 64, LDS, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                                row_pos, nq, nkv, window, scale, n_splits,
+                                                                                head_groups, part, out, *terms);
+      TL_LAUNCH_CHECK("attn_decode_ring with terms");
+      if (n_splits > 1) {
+        attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out, terms->gate);
+        TL_LAUNCH_CHECK("attn_decode_combine");
+      }
+      return 0;
+    }
+  }
+  if (terms != nullptr) {         // more terms on the scores, other head sizes: the kernel that reads the pages into registers
     if (d == DPAD)
       attn_decode_kernel<DPAD, true, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
                                                                             row_pos, nq, nkv, d, window, scale, n_splits,
@@ -1091,7 +1140,7 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
       }
       attn_decode_ring_kernel<DPAD, NS><<<grid, DC_WAVES * 64, LDS, st>>>(q, pages, table, table_stride, ring_pages,
                                                                           row_pos, nq, nkv, window, scale, n_splits,
-                                                                          head_groups, part, out);
+                                                                          head_groups, part, out, MoreTerms{});
       TL_LAUNCH_CHECK("attn_decode_ring");
       if (n_splits > 1) {
         attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);

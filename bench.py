@@ -53,7 +53,7 @@ def design_configs(z: dict, layers: int, share_from=None):
     Sozetar layers behind that index read its keys and values instead of making their own."""
     def mixer(i):
         m = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"],
-             "scale": z["dim"] ** -0.5, "q_temp": {"coef": 0.3, "every": 128}}
+             "scale": z["dim"] ** -0.5, "q_temp": {"coef": 0.25, "every": 256}}
         if z["window"]:
             m["mask"] = {"size": z["window"]}
         if share_from is not None and i > share_from:

@@ -627,3 +627,77 @@ def test_the_command_line_and_the_trace_replay(zoo, tmp_path):
     want = z["want"][2]
     assert rel_err(first, torch.stack([want[0], want[19], want[2]])) < TOL["float32"]
     assert rel_err(last, want[21:22]) < TOL["float32"]
+
+
+# ---------------------------------------------------------------------------------------------
+# the new parts in designs of other arrangements
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_new_parts_serve_other_designs(dtype):
+    """Two models that are neither design, from the registry's parts alone.  One: the output-norm block
+    around the older parts (attention without terms, SwiGLU, RMSNorm), which do not know of it.  Two: the
+    pre-norm block around the attention with a subset of its terms (a sink and a window: no biases, no
+    norm of q and k, no slopes, no gate, no factor on q), layer norm before the sublayers and a gelu gate."""
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.parts import LayerSpec, ModelSpec, PartSpec, Run
+    from torchless_rs_amd.weights import TensorDict, random_tensors
+    H, V, I, nq, nkv, d, L, eps, window = 64, 70, 96, 4, 2, 16, 2, 1e-5, 20
+    rms = PartSpec("rmsnorm", {"size": H, "eps": eps})
+    ln = PartSpec("layernorm", {"size": H, "eps": eps})
+    older = [LayerSpec(prefix=f"h.{i}.",
+                       mixer=PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                    "window": window, "position": PartSpec("none", {})}),
+                       ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}),
+                       mixer_norm=rms, ffn_norm=rms,
+                       block=PartSpec("output_norm", {"mixer_norm_name": "n1.", "ffn_norm_name": "n2."})) for i in range(L)]
+    subset = [LayerSpec(prefix=f"h.{i}.",
+                        mixer=PartSpec("scored_attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                            "window": window, "sink": True, "prefix": "self_attn."}),
+                        ffn=PartSpec("gated", {"hidden_size": H, "intermediate_size": I, "activation": "gelu_tanh"}),
+                        mixer_norm=ln, ffn_norm=ln,
+                        block=PartSpec("pre_norm", {"mixer_norm_name": "n1.", "ffn_norm_name": "n2."})) for i in range(L)]
+    ids = some_prompts(V, [45], seed=8)[0]
+
+    def lin(w, name, t):
+        return t @ w[name].double().T
+
+    for layers, final in ((older, rms), (subset, ln)):
+        spec = ModelSpec(hidden_size=H, vocab_size=V, embedding=PartSpec("tokens", {"vocab_size": V, "hidden_size": H}),
+                         embedding_prefix="model.", layers=layers, schedule=[Run(i) for i in range(L)],
+                         final_norm=final, final_norm_prefix="model.norm.",
+                         head=PartSpec("linear", {"vocab_size": V, "hidden_size": H}), head_prefix="lm_head.")
+        w = random_tensors(spec.weight_specs(), seed=4, std=0.2, norm_std=0.1, dtype=torch.bfloat16)
+        model = Model(spec, None, TORCH[dtype], torch.device("cuda:0"))
+        model.load_weights(TensorDict(w))
+        eng = Engine(model, max_tokens=256)
+        x = w["model.embed_tokens.weight"].double()[ids]
+        n = len(ids)
+        for i in range(L):
+            p = f"h.{i}."
+            if layers is older:
+                q, k, v = (lin(w, p + f"self_attn.{t}_proj.weight", x) for t in "qkv")
+                a = plain.attend(q.view(n, nq, d), k.view(n, nkv, d), v.view(n, nkv, d), d ** -0.5, None, None, window)
+                x = x + plain.rms_over_projection(lin(w, p + "self_attn.o_proj.weight", a.reshape(n, nq * d)),
+                                                  w[p + "n1.weight"].double(), eps)
+                g, u = lin(w, p + "mlp.gate_proj.weight", x), lin(w, p + "mlp.up_proj.weight", x)
+                x = x + plain.rms_over_projection(lin(w, p + "mlp.down_proj.weight", g / (1 + torch.exp(-g)) * u),
+                                                  w[p + "n2.weight"].double(), eps)
+            else:
+                y = plain.layer_norm(x, w[p + "n1.weight"].double(), eps)
+                q, k, v = (lin(w, p + f"self_attn.{t}", y) for t in "qkv")
+                a = plain.attend(q.view(n, nq, d), k.view(n, nkv, d), v.view(n, nkv, d), d ** -0.5, None,
+                                 w[p + "self_attn.sink"].double(), window)
+                x = x + lin(w, p + "self_attn.o", a.reshape(n, nq * d))
+                y = plain.layer_norm(x, w[p + "n2.weight"].double(), eps)
+                x = x + lin(w, p + "mlp.down_proj.weight",
+                            plain.gelu_tanh(lin(w, p + "mlp.gate_proj.weight", y)) * lin(w, p + "mlp.up_proj.weight", y))
+        nf = w["model.norm.weight"].double()
+        want = lin(w, "lm_head.weight", plain.rms_over_projection(x, nf, eps) if layers is older else plain.layer_norm(x, nf, eps))
+        s = eng.alloc()
+        got = [eng.step([SeqInput(s, ids[:30], list(range(30)))]).clone()]
+        got += [eng.step([SeqInput(s, [t], [0])]).clone() for t in ids[30:]]
+        eng.free(s)
+        close(torch.cat(got), want, dtype, "older parts in the new block" if layers is older else "a subset of the terms")
+        eng.close()

@@ -3,7 +3,8 @@ from .base import (ArchitectureEntry, ConfigError, ModelConfig, architecture_nam
                    registered_architectures, unregister_architecture)
 from .mistral import MistralConfig
 from .sozetar import SozetarConfig
+from .fanitar import FanitarConfig
 
-__all__ = ["ArchitectureEntry", "ConfigError", "ModelConfig", "MistralConfig", "SozetarConfig", "architecture_name",
+__all__ = ["ArchitectureEntry", "ConfigError", "ModelConfig", "MistralConfig", "SozetarConfig", "FanitarConfig", "architecture_name",
            "config_from_dict", "get_architecture", "load_config", "register_architecture",
            "registered_architectures", "unregister_architecture"]

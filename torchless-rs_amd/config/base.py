@@ -101,6 +101,19 @@ def load_config(model_dir: str) -> ModelConfig:
 
 # ---- helpers for config classes -------------------------------------------
 
+def take_obj(d, key, where, required=False) -> Optional[Dict[str, Any]]:
+    """The object under `key` (None if absent or null and not `required`); `where` names the
+    place in the file for the error."""
+    v = d.get(key)
+    if v is None:
+        if required:
+            raise ConfigError(f"config.json: {where} has no {key!r}")
+        return None
+    if not isinstance(v, dict):
+        raise ConfigError(f"config.json: {where}: {key!r} must be an object, got {v!r}")
+    return v
+
+
 def take_int(d, key, default=None, required=False, minimum=None, allow_none=False) -> Optional[int]:
     if key not in d or (d[key] is None and not allow_none and default is not None):
         if required:

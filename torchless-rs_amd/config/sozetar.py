@@ -18,21 +18,10 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
-from .base import ConfigError, ModelConfig, take_float, take_int
+from .base import ConfigError, ModelConfig, take_float, take_int, take_obj as _obj
 
 MAX_HEAD_DIM = 256          # the largest head the attention kernels take
 NAME = "Sozetar"
-
-
-def _obj(d, key, where, required=False) -> Optional[Dict[str, Any]]:
-    v = d.get(key)
-    if v is None:
-        if required:
-            raise ConfigError(f"config.json: {where} has no {key!r}")
-        return None
-    if not isinstance(v, dict):
-        raise ConfigError(f"config.json: {where}: {key!r} must be an object, got {v!r}")
-    return v
 
 
 @dataclass

@@ -14,15 +14,15 @@ void set_error(const char* fmt, ...) {
   va_end(ap);
 }
 
-// ---- embedding: out[n, :] = table[ids[n], :] (no scaling) -------------------
-// src/model/modules/embedding.rs:15-21 of the reference.
+// ---- embedding: out[n, :] = table[ids[n], :] * scale ---------------------------
+// src/model/modules/embedding.rs:15-21 of the reference (which has no scaling: scale 1).
 template <typename T>
-__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, int H,
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, int H, float scale,
                              float* __restrict__ out) {
   const int n = blockIdx.x;
   const T* row = table + (size_t)ids[n] * H;
   float* o = out + (size_t)n * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]);
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_f32(row[i]) * scale;
 }
 
 // ---- RMSNorm: y = x / sqrt(mean(x^2) + eps) * w ------------------------------
@@ -430,9 +430,22 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
 // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
 constexpr int ACT_SILU = 0;
 constexpr int ACT_GELU_TANH = 1;
+constexpr int ACT_SWISH_CLAMPED = 2;   // g' = min(g, limit), u' = clamp(u, -limit, limit): g' logistic(alpha g') (u' + shift)
 __device__ __forceinline__ float gate_act(float g, int act) {
   if (act == ACT_GELU_TANH) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
   return g / (1.0f + expf(-g));
+}
+// act(gate) * up with the constants of the functions that have some
+struct ActConstants {
+  float alpha, limit, shift;
+};
+__device__ __forceinline__ float gate_times_up(float g, float u, int act, ActConstants k) {
+  if (act == ACT_SWISH_CLAMPED) {
+    g = fminf(g, k.limit);
+    u = fminf(fmaxf(u, -k.limit), k.limit);
+    return (g / (1.0f + expf(-k.alpha * g))) * (u + k.shift);
+  }
+  return gate_act(g, act) * u;
 }
 
 // ---- h = silu(gate) * up, silu(g) = g / (1 + exp(-g)) ------------------------
@@ -450,7 +463,7 @@ __global__ void silu_mul_kernel(const float* __restrict__ gu, int I, TO* __restr
 // gu[n, 2I] in bfloat16 with columns in groups of 64 (32 of gate, then the 32 of up
 // that belong to them); out[n, I] = silu(gate) * up.  A thread takes 8 pairs.
 __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chunks, int I,
-                                      bf16* __restrict__ out, int act = ACT_SILU) {
+                                      bf16* __restrict__ out, int act = ACT_SILU, ActConstants k = ActConstants{1.f, 0.f, 0.f}) {
   const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= chunks) return;
   const int per_row = I / 8;
@@ -463,7 +476,7 @@ __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chu
 #pragma unroll
   for (int t = 0; t < 8; ++t) {
     const float gv = (float)g[t];
-    o[t] = (bf16)(gate_act(gv, act) * (float)u[t]);
+    o[t] = (bf16)gate_times_up(gv, (float)u[t], act, k);
   }
   *reinterpret_cast<bf16x8*>(out + n * I + group * 32 + part * 8) = o;
 }
@@ -567,11 +580,55 @@ __global__ void cast_rows_kernel(const float* __restrict__ x, size_t total, bf16
 
 // h = act(gate) * up from gu[n, 2I] = [gate | up]
 template <typename TO>
-__global__ void act_mul_kernel(const float* __restrict__ gu, int I, int act, TO* __restrict__ out) {
+__global__ void act_mul_kernel(const float* __restrict__ gu, int I, int act, ActConstants k, TO* __restrict__ out) {
   const int n = blockIdx.x;
   const float* row = gu + (size_t)n * 2 * I;
   for (int i = threadIdx.x; i < I; i += blockDim.x)
-    out[(size_t)n * I + i] = from_f32<TO>(gate_act(row[i], act) * row[I + i]);
+    out[(size_t)n * I + i] = from_f32<TO>(gate_times_up(row[i], row[I + i], act, k));
+}
+
+// ---- an RMS norm of a sublayer's OUTPUT, added to the stream ---------------------------------
+// x += z / sqrt(mean(z^2) + eps) * w.  With `w_next`, the norm that reads the stream next runs on
+// the new row at once: out = x / sqrt(mean(x^2) + eps_next) * w_next (the row is read where it
+// was just written, by the thread that wrote it).
+template <typename TO>
+__global__ void __launch_bounds__(256)
+rmsnorm_add_kernel(const float* __restrict__ z, const float* __restrict__ w, float eps, float* __restrict__ x,
+                   const float* __restrict__ w_next, float eps_next, TO* __restrict__ out, int H) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x;
+  const float* zr = z + (size_t)n * H;
+  float* xr = x + (size_t)n * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) ss += zr[i] * zr[i];
+  ss = block_sum<256>(ss, sh);
+  const float rms = sqrtf(ss / (float)H + eps);
+  float s2 = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    const float t = xr[i] + (zr[i] / rms) * w[i];
+    xr[i] = t;
+    s2 += t * t;
+  }
+  if (w_next == nullptr) return;
+  s2 = block_sum<256>(s2, sh);
+  const float rms2 = sqrtf(s2 / (float)H + eps_next);
+  TO* o = out + (size_t)n * H;
+  for (int i = threadIdx.x; i < H; i += 256) o[i] = from_f32<TO>((xr[i] / rms2) * w_next[i]);
+}
+
+// x[n, :] += extra[n, :] (may be null) + vec[:]: what a pass over a run of layers adds at its start
+__global__ void stream_entry_kernel(float* __restrict__ x, const float* __restrict__ extra,
+                                    const float* __restrict__ vec, int H, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float t = x[i];
+  if (extra) t += extra[i];
+  x[i] = t + vec[i % H];
+}
+
+__global__ void scale_kernel(float* __restrict__ x, float s, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) x[i] *= s;
 }
 
 // tokens[j] = src[idx[j]]: the ids that the sampler left on the device become the next step's
@@ -603,15 +660,15 @@ extern "C" {
 const char* tl_last_error() { return g_err; }
 int tl_page_size() { return PAGE; }      // what this library was compiled with (csrc/page.h)
 
-int tl_embed(const void* table, int table_dt, const int* ids, int n, int H, float* out,
+int tl_embed(const void* table, int table_dt, const int* ids, int n, int H, float scale, float* out,
              hipStream_t st) {
   TL_REQUIRE(n >= 0 && H > 0, "embed: bad sizes n=%d H=%d", n, H);
   if (n == 0) return 0;
   const int nt = H >= 256 ? 256 : 64;
   if (table_dt == DT_F32)
-    embed_kernel<float><<<n, nt, 0, st>>>((const float*)table, ids, H, out);
+    embed_kernel<float><<<n, nt, 0, st>>>((const float*)table, ids, H, scale, out);
   else if (table_dt == DT_BF16)
-    embed_kernel<bf16><<<n, nt, 0, st>>>((const bf16*)table, ids, H, out);
+    embed_kernel<bf16><<<n, nt, 0, st>>>((const bf16*)table, ids, H, scale, out);
   else
     TL_REQUIRE(false, "embed: unknown dtype code %d", table_dt);
   TL_LAUNCH_CHECK("embed");
@@ -910,14 +967,17 @@ int tl_cast_rows(const float* x, long long total, void* out, hipStream_t st) {
   return 0;
 }
 
-int tl_act_mul(const float* gu, int n, int I, int act, void* out, int out_dt, hipStream_t st) {
+int tl_act_mul(const float* gu, int n, int I, int act, float alpha, float limit, float shift, void* out, int out_dt,
+               hipStream_t st) {
   TL_REQUIRE(n >= 0 && I > 0, "act_mul: bad sizes n=%d I=%d", n, I);
-  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH, "act_mul: no function of code %d", act);
+  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMPED, "act_mul: no function of code %d", act);
+  TL_REQUIRE(act != ACT_SWISH_CLAMPED || limit > 0.f, "act_mul: the clamp needs a positive limit");
   if (n == 0) return 0;
+  const ActConstants k{alpha, limit, shift};
   if (out_dt == DT_F32)
-    act_mul_kernel<float><<<n, 256, 0, st>>>(gu, I, act, (float*)out);
+    act_mul_kernel<float><<<n, 256, 0, st>>>(gu, I, act, k, (float*)out);
   else if (out_dt == DT_BF16)
-    act_mul_kernel<bf16><<<n, 256, 0, st>>>(gu, I, act, (bf16*)out);
+    act_mul_kernel<bf16><<<n, 256, 0, st>>>(gu, I, act, k, (bf16*)out);
   else
     TL_REQUIRE(false, "act_mul: unknown dtype code %d", out_dt);
   TL_LAUNCH_CHECK("act_mul");
@@ -925,15 +985,50 @@ int tl_act_mul(const float* gu, int n, int I, int act, void* out, int out_dt, hi
 }
 
 // tl_silu_mul_pairs with the gate's function chosen (codes as tl_act_mul)
-int tl_act_mul_pairs(const void* gu, int n, int I, int act, void* out, hipStream_t st) {
+int tl_act_mul_pairs(const void* gu, int n, int I, int act, float alpha, float limit, float shift, void* out,
+                     hipStream_t st) {
   TL_REQUIRE(n >= 0 && I > 0 && I % 32 == 0, "act_mul_pairs: bad sizes n=%d I=%d (I in steps of 32)", n, I);
-  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH, "act_mul_pairs: no function of code %d", act);
+  TL_REQUIRE(act == ACT_SILU || act == ACT_GELU_TANH || act == ACT_SWISH_CLAMPED, "act_mul_pairs: no function of code %d", act);
   TL_REQUIRE((uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0, "act_mul_pairs: buffers must be 16-byte aligned");
   if (n == 0) return 0;
   const long long chunks = (long long)n * (I / 8);
   TL_REQUIRE((chunks + 255) / 256 < 2147483647LL, "act_mul_pairs: too many elements");
-  silu_mul_pairs_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const bf16*)gu, chunks, I, (bf16*)out, act);
+  silu_mul_pairs_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const bf16*)gu, chunks, I, (bf16*)out, act,
+                                                                          ActConstants{alpha, limit, shift});
   TL_LAUNCH_CHECK("act_mul_pairs");
+  return 0;
+}
+
+// x += rmsnorm(z; w, eps); with w_next also out = rmsnorm(x; w_next, eps_next)
+int tl_rmsnorm_add(const float* z, const float* w, float eps, float* x, const float* w_next, float eps_next, void* out,
+                   int out_dt, int n, int H, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && z && w && x, "rmsnorm_add: bad arguments n=%d H=%d", n, H);
+  TL_REQUIRE(w_next == nullptr || (out != nullptr && (out_dt == DT_F32 || out_dt == DT_BF16)),
+             "rmsnorm_add: the norm that follows needs a buffer of a known type");
+  if (n == 0) return 0;
+  if (w_next == nullptr || out_dt == DT_F32)
+    rmsnorm_add_kernel<float><<<n, 256, 0, st>>>(z, w, eps, x, w_next, eps_next, (float*)out, H);
+  else
+    rmsnorm_add_kernel<bf16><<<n, 256, 0, st>>>(z, w, eps, x, w_next, eps_next, (bf16*)out, H);
+  TL_LAUNCH_CHECK("rmsnorm_add");
+  return 0;
+}
+
+// x[n, H] += extra[n, H] (may be null) + vec[H]
+int tl_stream_entry(float* x, const float* extra, const float* vec, int n, int H, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && x && vec, "stream_entry: bad arguments n=%d H=%d", n, H);
+  if (n == 0) return 0;
+  const size_t total = (size_t)n * H;
+  stream_entry_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, extra, vec, H, total);
+  TL_LAUNCH_CHECK("stream_entry");
+  return 0;
+}
+
+int tl_scale(float* x, float s, long long total, hipStream_t st) {
+  TL_REQUIRE(total >= 0 && x, "scale: bad arguments");
+  if (total == 0) return 0;
+  scale_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, s, (size_t)total);
+  TL_LAUNCH_CHECK("scale");
   return 0;
 }
 

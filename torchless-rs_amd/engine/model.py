@@ -31,7 +31,11 @@ class Model:
                        for ls in spec.layers]
         self.final_norm = make_part("norm", spec.final_norm)
         self.head = make_part("head", spec.head)
+        self.stream_parts = [make_part("stream", sp) for _, sp in spec.stream_parts]
         for i, run in enumerate(spec.schedule):
+            if run.entry is not None and not (0 <= run.entry[0] < len(self.stream_parts)):
+                raise ValueError(f"schedule entry {i} names stream part {run.entry[0]}, there are "
+                                 f"{len(self.stream_parts)}")
             if not (0 <= run.layer < len(self.blocks)):
                 raise ValueError(f"schedule entry {i} names layer {run.layer}, there are "
                                  f"{len(self.blocks)}")
@@ -39,18 +43,19 @@ class Model:
                 raise ValueError(f"schedule entry {i} reads the cache of entry {run.kv_from}, which "
                                  "is not an earlier one")
         self.loaded = False
-        self.graph_safe = all(p.graph_safe for p in [self.embedding, self.final_norm, self.head] + self.blocks)
+        self.graph_safe = all(p.graph_safe for p in self._all_parts())
+
+    def _all_parts(self):
+        return [self.embedding, self.final_norm, self.head] + self.blocks + self.stream_parts
 
     def may_capture(self, n_rows: int) -> bool:
         """May a single-token step of `n_rows` rows be captured as a graph and replayed?  Every
         part answers for itself; the step function knows nothing of their kernels."""
-        return self.loaded and all(p.may_capture(n_rows)
-                                   for p in [self.embedding, self.final_norm, self.head] + self.blocks)
+        return self.loaded and all(p.may_capture(n_rows) for p in self._all_parts())
 
     def prefers_eager(self, n_new, len_before, device) -> bool:
         """Does any part want to shape its launches by this step's own lengths (see `Part.prefers_eager`)?"""
-        return any(p.prefers_eager(n_new, len_before, device)
-                   for p in [self.embedding, self.final_norm, self.head] + self.blocks)
+        return any(p.prefers_eager(n_new, len_before, device) for p in self._all_parts())
 
     # ---- weights -----------------------------------------------------------
     def load_weights(self, source, tiled_copies: bool = True) -> None:
@@ -71,6 +76,8 @@ class Model:
         self.embedding.load(sub(spec.embedding_prefix), self.dtype)
         for ls, blk in zip(spec.layers, self.blocks):
             blk.load(sub(ls.prefix), self.dtype)
+        for (prefix, _), part in zip(spec.stream_parts, self.stream_parts):
+            part.load(sub(prefix), self.dtype)
         self.final_norm.load(sub(spec.final_norm_prefix), self.dtype)
         head_t = sub(spec.head_prefix)
         head_t["__embedding__"] = getattr(self.embedding, "table", None)
@@ -129,9 +136,22 @@ class Model:
         ws = ctx.workspace
         x = ws.get("residual", (ctx.n_rows, H), torch.float32)
         self.embedding.forward(ctx, ctx.tokens, x)
-        order = [self.blocks[run.layer] for run in self.spec.schedule]
+        embedded = None
+        if any(p.needs_embedding for p in self.stream_parts):      # someone adds the embedding's output again later
+            embedded = ws.get("embedded", (ctx.n_rows, H), torch.float32)
+            self.embedding.forward(ctx, ctx.tokens, embedded)
+        schedule = self.spec.schedule
+        order = [self.blocks[run.layer] for run in schedule]
         for i, (block, binding) in enumerate(zip(order, runs)):
-            after = order[i + 1].entry_norm() if i + 1 < len(order) and hasattr(order[i + 1], "entry_norm") else None
+            if schedule[i].entry is not None:
+                part, t = schedule[i].entry
+                flush_pending(ctx, x)
+                ctx.prenormed = None
+                self.stream_parts[part].forward(ctx, x, embedded, t)
+            # the norm that reads the stream next, unless the stream changes before it does
+            after = (order[i + 1].entry_norm()
+                     if i + 1 < len(order) and hasattr(order[i + 1], "entry_norm") and schedule[i + 1].entry is None
+                     else None)
             if after is not None:
                 block.forward(ctx, binding, x, norm_after=after)
             else:

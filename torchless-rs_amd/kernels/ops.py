@@ -78,13 +78,48 @@ def _req(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
     raise KernelError(f"{name}: shape {tuple(t.shape)}, kernel needs {tuple(shape)}")
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """out[n, :] = table[ids[n], :] widened to float32."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """out[n, :] = table[ids[n], :] widened to float32, times `scale`."""
     n, H = ids.shape[0], table.shape[1]
     _req(table, "embed.table")
     _req(ids, "embed.ids", torch.int32, (n,))
     _req(out, "embed.out", torch.float32, (n, H))
-    _check(lib().tl_embed(_p(table), _code(table.dtype), _p(ids), n, H, _p(out), _stream()))
+    _check(lib().tl_embed(_p(table), _code(table.dtype), _p(ids), n, H, ctypes.c_float(scale), _p(out), _stream()))
+
+
+def rmsnorm_add(z: torch.Tensor, w: torch.Tensor, eps: float, x: torch.Tensor, w_next: Optional[torch.Tensor] = None,
+                eps_next: float = 0.0, out: Optional[torch.Tensor] = None) -> None:
+    """The RMS norm of a sublayer's output added to the stream: x += z / sqrt(mean(z^2) + eps) * w
+    (z, x float32 [n, H]).  With `w_next` the norm that reads the stream next runs in the same
+    kernel: out = x / sqrt(mean(x^2) + eps_next) * w_next, in `out`'s dtype."""
+    n, H = z.shape
+    _req(z, "rmsnorm_add.z", torch.float32)
+    _req(w, "rmsnorm_add.w", torch.float32, (H,))
+    _req(x, "rmsnorm_add.x", torch.float32, (n, H))
+    if w_next is not None:
+        _req(w_next, "rmsnorm_add.w_next", torch.float32, (H,))
+        if out is None:
+            raise KernelError("rmsnorm_add: the norm that follows needs `out`")
+        _req(out, "rmsnorm_add.out", None, (n, H))
+    _check(lib().tl_rmsnorm_add(_p(z), _p(w), ctypes.c_float(eps), _p(x), _p(w_next), ctypes.c_float(eps_next),
+                                _p(out) if w_next is not None else None,
+                                _code(out.dtype) if w_next is not None else DT_F32, n, H, _stream()))
+
+
+def stream_entry(x: torch.Tensor, extra: Optional[torch.Tensor], vec: torch.Tensor) -> None:
+    """x[n, :] += extra[n, :] (None: nothing) + vec[:], all float32."""
+    n, H = x.shape
+    _req(x, "stream_entry.x", torch.float32)
+    if extra is not None:
+        _req(extra, "stream_entry.extra", torch.float32, (n, H))
+    _req(vec, "stream_entry.vec", torch.float32, (H,))
+    _check(lib().tl_stream_entry(_p(x), _p(extra), _p(vec), n, H, _stream()))
+
+
+def scale_(x: torch.Tensor, s: float) -> None:
+    """x *= s (float32, in place)."""
+    _req(x, "scale.x", torch.float32)
+    _check(lib().tl_scale(_p(x), ctypes.c_float(s), ctypes.c_longlong(x.numel()), _stream()))
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor) -> None:
@@ -295,7 +330,7 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().tl_silu_mul(_p(gu), n, I2 // 2, _p(out), _code(out.dtype), _stream()))
 
 
-def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu", constants=None) -> None:
     """The same on bfloat16 gu whose columns come in groups of 64: 32 of gate,
     then the 32 of up that belong to them (`interleave_pairs`); `activation`: the gate's
     function (`ACTIVATIONS`)."""
@@ -307,7 +342,8 @@ def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu"
         return
     if activation not in ACTIVATIONS:
         raise KernelError(f"silu_mul_pairs: no function {activation!r}; there are {sorted(ACTIVATIONS)}")
-    _check(lib().tl_act_mul_pairs(_p(gu), n, I2 // 2, ACTIVATIONS[activation], _p(out), _stream()))
+    _check(lib().tl_act_mul_pairs(_p(gu), n, I2 // 2, ACTIVATIONS[activation], *_act_constants(activation, constants),
+                                  _p(out), _stream()))
 
 
 def layernorm(z: torch.Tensor, w: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
@@ -338,17 +374,31 @@ def cast_rows(x: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().tl_cast_rows(_p(x), ctypes.c_longlong(x.numel()), _p(out), _stream()))
 
 
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+# The functions of a gated feed-forward.  silu: g / (1 + e^-g); gelu_tanh: the tanh form of gelu;
+# swish_clamped, with the constants `alpha`, `limit` and `shift`: g' = min(g, limit),
+# u' = clamp(u, -limit, limit), and the hidden value is g' / (1 + e^(-alpha g')) * (u' + shift).
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swish_clamped": 2}
+ACTIVATION_CONSTANTS = {"swish_clamped": ("alpha", "limit", "shift")}
 
 
-def act_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
-    """out[n, i] = act(gu[n, i]) * gu[n, I + i]; act: silu, or gelu_tanh, the tanh form of gelu."""
+def _act_constants(activation: str, constants):
+    """(alpha, limit, shift) as the kernels take them; a function without constants ignores them."""
+    names = ACTIVATION_CONSTANTS.get(activation, ())
+    given = dict(constants or {})
+    if set(given) != set(names):
+        raise KernelError(f"activation {activation!r} takes the constants {sorted(names)}, got {sorted(given)}")
+    return tuple(ctypes.c_float(float(given.get(k, 0.0))) for k in ("alpha", "limit", "shift"))
+
+
+def act_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu", constants=None) -> None:
+    """out[n, i] = act(gu[n, i]) * gu[n, I + i]; act: one of `ACTIVATIONS`, `constants` its constants."""
     n, I2 = gu.shape
     if activation not in ACTIVATIONS:
         raise KernelError(f"act_mul: no function {activation!r}; there are {sorted(ACTIVATIONS)}")
     _req(gu, "act_mul.gu", torch.float32)
     _req(out, "act_mul.out", None, (n, I2 // 2))
-    _check(lib().tl_act_mul(_p(gu), n, I2 // 2, ACTIVATIONS[activation], _p(out), _code(out.dtype), _stream()))
+    _check(lib().tl_act_mul(_p(gu), n, I2 // 2, ACTIVATIONS[activation], *_act_constants(activation, constants),
+                            _p(out), _code(out.dtype), _stream()))
 
 
 class ScoreTerms:
@@ -511,6 +561,108 @@ def kv_commit_wide(k: torch.Tensor, v: torch.Tensor, row_seq, row_pos, len_after
                                    table.shape[1], ring_pages, n, nkv, dk, dv, _p(pages), _stream()))
 
 
+def latent_norms(proj: torch.Tensor, na: int, nb: int, wa: torch.Tensor, wb: torch.Tensor, eps: float, a: torch.Tensor,
+                 b: torch.Tensor, gate: Optional[torch.Tensor]) -> None:
+    """proj float32 [n, na + nb + ng] = [a | b | g]: a and b each divided by their root mean square
+    (eps inside the root) and multiplied by their weights (float32 [na], [nb]) into the compute dtype;
+    `gate` (float32 [n, ng], or None when ng = 0) = the logistic function of g."""
+    n, width = proj.shape
+    ng = width - na - nb
+    _req(proj, "latent_norms.proj", torch.float32)
+    _req(wa, "latent_norms.wa", torch.float32, (na,))
+    _req(wb, "latent_norms.wb", torch.float32, (nb,))
+    _req(a, "latent_norms.a", None, (n, na))
+    _req(b, "latent_norms.b", a.dtype, (n, nb))
+    if ng < 0 or (ng > 0) != (gate is not None):
+        raise KernelError(f"latent_norms: a row of {width} holds {na} + {nb} and {ng} gate channels; gate buffer "
+                          f"{'given' if gate is not None else 'missing'}")
+    if gate is not None:
+        _req(gate, "latent_norms.gate", torch.float32, (n, ng))
+    _check(lib().tl_latent_norms(_p(proj), n, na, nb, ng, _p(wa), _p(wb), ctypes.c_float(eps), _p(a), _p(b), _p(gate),
+                                 _code(a.dtype), _stream()))
+
+
+def split_heads(qf: torch.Tensor, kvf: torch.Tensor, row_pos, nq: int, nkv: int, dk: int, dv: int, q: torch.Tensor,
+                k, v, table=None, ring_pages: int = 0, pages=None) -> None:
+    """qf float32 [n, nq*dk] and kvf float32 [n, nkv*dk + nkv*dv] (keys of all heads, then values of all
+    heads) -> q [n, nq, dk], k [n, nkv, dk] and v [n, nkv, dv] in the compute dtype; or, with `pages`
+    (one token a sequence, row n belongs to sequence n), k and v straight into the page of the row's
+    position."""
+    n = qf.shape[0]
+    _req(qf, "split_heads.qf", torch.float32, (n, nq * dk))
+    _req(kvf, "split_heads.kvf", torch.float32, (n, nkv * (dk + dv)))
+    _req(row_pos, "split_heads.row_pos", torch.int32, (n,))
+    _req(q, "split_heads.q", None, (n, nq, dk))
+    stride = 0
+    if pages is None:
+        _req(k, "split_heads.k", q.dtype, (n, nkv, dk))
+        _req(v, "split_heads.v", q.dtype, (n, nkv, dv))
+    else:
+        _req_pages(pages, nkv, dk, dv, "split_heads")
+        _req(table, "split_heads.table", torch.int32)
+        if pages.dtype != q.dtype or table.dim() != 2 or table.shape[0] != n:
+            raise KernelError("split_heads: pages of q's dtype and a page table with one row per row")
+        stride = table.shape[1]
+    kv = kvf.data_ptr()
+    _check(lib().tl_split_heads(_p(qf), nq * dk, ctypes.c_void_p(kv), ctypes.c_void_p(kv + 4 * nkv * dk),
+                                nkv * (dk + dv), _p(row_pos), n, nq, nkv, dk, dv, _p(q),
+                                _p(k) if pages is None else None, _p(v) if pages is None else None, _code(q.dtype),
+                                _p(table), stride, int(ring_pages), _p(pages), _stream()))
+
+
+def mul_gate(x: torch.Tensor, gate: torch.Tensor) -> None:
+    """x *= gate, element by element (x in the compute dtype, gate float32 of as many elements)."""
+    _req(x, "mul_gate.x")
+    _req(gate, "mul_gate.gate", torch.float32)
+    if gate.numel() != x.numel():
+        raise KernelError(f"mul_gate: {x.numel()} values and {gate.numel()} gates")
+    _check(lib().tl_mul_gate(_p(x), _p(gate), ctypes.c_longlong(x.numel()), _code(x.dtype), _stream()))
+
+
+def diff_split(proj: torch.Tensor, bias, row_pos, rotation, H: int, G: int, d: int, dv: int, q: torch.Tensor, k, v,
+               table=None, ring_pages: int = 0, pages=None) -> None:
+    """A row of the fused projection of a differential attention, float32 [n, 2*H*d + 2*G*d + G*dv] =
+    [q | k | v] with two maps of d channels per head, plus `bias` (float32 over the row, or None);
+    each map of q and k rotated (`rotation`: the first channels of every MAP); q laid out as 2*H heads
+    of 2*d channels, map m of head h as head 2h + m with its channels in half m and zeros in the
+    other; k [n, G, 2*d] and v [n, G, dv] as rows, or, with `pages` (one token a sequence), straight
+    into the page of the row's position."""
+    n = proj.shape[0]
+    rot = _rotation(rotation, d, "diff_split")
+    _req(proj, "diff_split.proj", torch.float32, (n, 2 * H * d + 2 * G * d + G * dv))
+    if bias is not None:
+        _req(bias, "diff_split.bias", torch.float32, (proj.shape[1],))
+    _req(row_pos, "diff_split.row_pos", torch.int32, (n,))
+    _req(q, "diff_split.q", None, (n, 2 * H, 2 * d))
+    stride = 0
+    if pages is None:
+        _req(k, "diff_split.k", q.dtype, (n, G, 2 * d))
+        _req(v, "diff_split.v", q.dtype, (n, G, dv))
+    else:
+        _req_pages(pages, G, 2 * d, dv, "diff_split")
+        _req(table, "diff_split.table", torch.int32)
+        if pages.dtype != q.dtype or table.dim() != 2 or table.shape[0] != n:
+            raise KernelError("diff_split: pages of q's dtype and a page table with one row per row")
+        stride = table.shape[1]
+    if rot.interleaved:
+        raise KernelError("diff_split: pairs (2i, 2i + 1) are not served, only (i, i + rotary_dim / 2)")
+    _check(lib().tl_diff_split(_p(proj), _p(bias), _p(row_pos), _p(rot.inv_freq), rot.rotary_dim, n, H, G, d, dv, _p(q),
+                               _p(k) if pages is None else None, _p(v) if pages is None else None, _code(q.dtype),
+                               _p(table), stride, int(ring_pages), _p(pages), _stream()))
+
+
+def diff_combine(att: torch.Tensor, lam: float, eps: float, post: float, out: torch.Tensor) -> None:
+    """att [n, 2*H, dv] (heads 2h and 2h + 1: the two maps of head h) -> out [n, H, dv]:
+    o = a1 - lam * a2, then o / sqrt(mean(o^2) + eps) * post, in float32."""
+    n, H2, dv = att.shape
+    _req(att, "diff_combine.att")
+    if H2 % 2:
+        raise KernelError(f"diff_combine: {H2} maps are not pairs")
+    _req(out, "diff_combine.out", att.dtype, (n, H2 // 2, dv))
+    _check(lib().tl_diff_combine(_p(att), n, H2 // 2, dv, ctypes.c_float(lam), ctypes.c_float(eps), ctypes.c_float(post),
+                                 _p(out), _code(att.dtype), _stream()))
+
+
 def take_tokens(src: torch.Tensor, idx: torch.Tensor, vocab: int, tokens: torch.Tensor) -> None:
     """tokens[j] = src[idx[j]] (int32, on the device); ids outside [0, vocab) become 0."""
     n = tokens.shape[0]
@@ -556,10 +708,13 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, s
 EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR, EPI_GELU_PAIR = 0, 1, 2, 3
 
 
+PAIR_EPILOGUES = ("silu", "gelu_tanh")       # the gate functions that the products' paired epilogue knows
+
+
 def _pair_epilogue(pair_act: str) -> int:
     """The code of the paired epilogue act(gate) * up for the gate's function `pair_act`."""
-    if pair_act not in ACTIVATIONS:
-        raise KernelError(f"paired epilogue: no function {pair_act!r}; there are {sorted(ACTIVATIONS)}")
+    if pair_act not in PAIR_EPILOGUES:
+        raise KernelError(f"paired epilogue: no function {pair_act!r}; there are {sorted(PAIR_EPILOGUES)}")
     return EPI_GELU_PAIR if pair_act == "gelu_tanh" else EPI_SILU_PAIR
 
 

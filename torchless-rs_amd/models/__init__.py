@@ -5,6 +5,7 @@ from ..parts import base as _parts_base
 from .. import parts as _parts            # registers the parts
 from . import mistral as _mistral         # registers MistralForCausalLM
 from . import sozetar as _sozetar         # registers Sozetar
+from . import fanitar as _fanitar         # registers Fanitar
 
 
 def model_spec_for(cfg: ModelConfig):

@@ -1,7 +1,8 @@
 from .base import (FeedForward, LayerSpec, Mixer, ModelSpec, Norm, Part, PartSpec, Position, Run,
                    RunBinding, StepContext, Workspace, make_part, register_part, registered_parts,
                    unregister_part)
-from . import attention, attention_scored, block, embedding, ffn, norms, position   # noqa: F401  (register)
+from . import (attention, attention_diff, attention_latent, attention_scored, block, embedding, ffn, norms,   # noqa: F401
+               position)
 from .linear import Linear
 
 __all__ = ["FeedForward", "LayerSpec", "Linear", "Mixer", "ModelSpec", "Norm", "Part", "PartSpec",

@@ -215,4 +215,30 @@ class ScoredAttentionMixer(Mixer):
         ops.add_partials(x, z.view(1, *z.shape))
 
 
+def attend_and_commit(ctx, run, q: torch.Tensor, k, v, nkv: int, dk: int, dv: int, terms, gate, att: torch.Tensor,
+                      tag: str = "") -> None:
+    """The attention of a step for a mixer that owns its keys and values and has made q [n, nq, dk]
+    and, unless every sequence brings one token (k and v are then None and lie in their pages
+    already), this step's k [n, nkv, dk] and v [n, nkv, dv]: the step's rows attend to the pages
+    for cached positions and to k and v for the new ones (values transposed by tiles where the
+    matrix cores run), and k and v are committed to the pages afterwards."""
+    group = run.kv_group
+    pages = group.storage[run.kv_layer]
+    table = ctx.tables[run.kv_group_index]
+    if ctx.all_single:
+        ops.attention_scored(q, None, None, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_after, terms, gate, att)
+        return
+    vt = None
+    if ops.scored_on_matrix_cores(ctx.dtype, dk, dv):
+        vt = ctx.workspace.get("attend_vt" + tag, (nkv, dv, ctx.host["aligned_cols"]), ctx.dtype)
+        ops.v_tiles_rows(v, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, ctx.len_after)
+    ops.attention_scored(q, k, v, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_before, terms, gate, att,
+                         vt_new=vt)
+    if vt is not None and pages.dim() == 5:       # values a tile at a time, in whole lines
+        ops.kv_commit_tiles(k, vt, ctx.row_seq, ctx.row_pos, ctx.tile_off, ctx.len_before, ctx.len_after, table,
+                            group.ring_pages, pages)
+    else:
+        ops.kv_commit_wide(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table, group.ring_pages, pages)
+
+
 register_part("mixer", "scored_attention", ScoredAttentionMixer)

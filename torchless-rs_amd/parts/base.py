@@ -24,7 +24,7 @@ import torch
 
 from ..weights.binding import WeightSpec
 
-CATEGORIES = ("mixer", "ffn", "norm", "position", "block", "embedding", "head")
+CATEGORIES = ("mixer", "ffn", "norm", "position", "block", "embedding", "head", "stream")
 _PARTS: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
 
 
@@ -64,14 +64,20 @@ class LayerSpec:
     mixer_norm: PartSpec
     ffn_norm: Optional[PartSpec]
     block: PartSpec = field(default_factory=lambda: PartSpec("pre_norm"))
+    # norms of the sublayers' OUTPUTS, for arrangements that norm on both sides of a sublayer
+    mixer_out_norm: Optional[PartSpec] = None
+    ffn_out_norm: Optional[PartSpec] = None
 
 
 @dataclass
 class Run:
     """One entry of the schedule: run `layer`; `kv_from`, if set, is the index
-    of an earlier entry whose cache this run reads instead of owning one."""
+    of an earlier entry whose cache this run reads instead of owning one;
+    `entry`, if set, is (index into `ModelSpec.stream_parts`, t): that part changes
+    the stream right before this run, as its t-th call of the step."""
     layer: int
     kv_from: Optional[int] = None
+    entry: Optional[Tuple[int, int]] = None
 
 
 @dataclass
@@ -87,6 +93,8 @@ class ModelSpec:
     head: PartSpec
     head_prefix: str
     ignore_tensors: Tuple[str, ...] = ()
+    # parts of category "stream" that change the stream between runs (`Run.entry`): (name prefix, spec)
+    stream_parts: List[Tuple[str, PartSpec]] = field(default_factory=list)
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         """Every tensor name the model binds, in a fixed order."""
@@ -97,6 +105,9 @@ class ModelSpec:
             blk = make_part("block", PartSpec(ls.block.kind, dict(ls.block.params, layer=ls)))
             for k, v in blk.weight_specs().items():
                 out[ls.prefix + k] = v
+        for prefix, sp in self.stream_parts:
+            for k, v in make_part("stream", sp).weight_specs().items():
+                out[prefix + k] = v
         for k, v in make_part("norm", self.final_norm).weight_specs().items():
             out[self.final_norm_prefix + k] = v
         for k, v in make_part("head", self.head).weight_specs().items():
@@ -154,10 +165,13 @@ class Norm(Part):
         return None
 
     def add_to(self, ctx: "StepContext", z: torch.Tensor, x: torch.Tensor, out: Optional[torch.Tensor] = None,
-               bias: Optional[torch.Tensor] = None) -> None:
+               bias: Optional[torch.Tensor] = None, then=None) -> None:
         """The norm of a sublayer's output: x += norm(z + bias), z float32 [n, H] (`bias`: float32
         [H], what the sublayer's last product left to add); `out`, if given, receives the new x in
-        its dtype.  This is the plain way in three kernels; a norm with a kernel for it overrides."""
+        its dtype.  `then` = (norm, buffer) names the norm that reads the stream next: a norm whose
+        kernel can run that one on the new row as well does, and leaves `ctx.prenormed` = (norm,
+        buffer, None) for `read_through_norm`; any other ignores it.  This is the plain way in
+        three kernels; a norm with a kernel for it overrides."""
         from ..kernels import ops
         if bias is not None:
             z += bias
@@ -169,6 +183,16 @@ class Norm(Part):
                 out.copy_(x)
             else:
                 ops.cast_rows(x, out)
+
+
+class StreamPart(Part):
+    """A part that changes the residual stream between two runs of the schedule (`Run.entry`)."""
+    needs_embedding = False       # True: `forward` is handed the embedding's output of this step
+
+    def forward(self, ctx: "StepContext", x: torch.Tensor, embedded: Optional[torch.Tensor], t: int) -> None:
+        """x: the stream, float32 [n, H], changed in place; `embedded`: the stream as the embedding
+        left it (None unless `needs_embedding`); t: which call of this part within the step."""
+        raise NotImplementedError
 
 
 class Position(Part):

@@ -1,8 +1,10 @@
 """The arrangements of a layer.  `PreNormBlock`: x += mixer(norm(x)); x += ffn(norm(x))
 (src/model/modules/layer.rs:28-56 of the reference).  `OutputNormBlock`: the
 sublayers read the stream itself and their OUTPUT is normed before the sum,
-x += norm(mixer(x)); x += norm(ffn(x)), the feed-forward being optional.  The
-residual stream x is float32 in both."""
+x += norm(mixer(x)); x += norm(ffn(x)), the feed-forward being optional.
+`SandwichNormBlock`: a norm on both sides of each sublayer,
+x += norm_b(mixer(norm_a(x))); x += norm_d(ffn(norm_c(x))).  The residual stream x
+is float32 in all."""
 from __future__ import annotations
 
 from typing import Dict, Optional
@@ -12,7 +14,7 @@ import torch
 from ..weights.binding import WeightSpec
 from ..kernels import ops
 from .base import (LayerSpec, Part, expect_norm, flush_pending, make_part, part_done, read_through_norm,
-                   register_part, splittable_entry)
+                   register_part, splittable_entry, take_row_factor)
 
 
 class PreNormBlock(Part):
@@ -144,5 +146,83 @@ class OutputNormBlock(Part):
             ctx.host["stream_copy"] = y
 
 
+class SandwichNormBlock(Part):
+    """x += out_norm1(mixer(norm1(x))); then, if the layer has a feed-forward,
+    x += out_norm2(ffn(norm2(x))).  The four norms are the layer's `mixer_norm`, `mixer_out_norm`,
+    `ffn_norm` and `ffn_out_norm`, bound under the four names given here.
+
+    A sublayer's result is stored (`produce`, or `forward` into a zeroed buffer) and the norm of
+    it is added to the stream by `Norm.add_to`, which is told the norm that reads the stream next
+    (the feed-forward's, or the next block's `entry_norm`): a norm that can run both in one kernel
+    leaves the second one's result for `read_through_norm`."""
+
+    def __init__(self, layer: LayerSpec, names=("norm1.", "norm1b.", "norm2.", "norm2b.")):
+        if layer.mixer_out_norm is None or (layer.ffn is not None and (layer.ffn_norm is None or layer.ffn_out_norm is None)):
+            raise ValueError("sandwich block: the layer names no norm for a sublayer's output (or input)")
+        self.mixer = make_part("mixer", layer.mixer)
+        self.mixer_norm = make_part("norm", layer.mixer_norm)
+        self.mixer_out_norm = make_part("norm", layer.mixer_out_norm)
+        self.ffn = make_part("ffn", layer.ffn) if layer.ffn is not None else None
+        self.ffn_norm = make_part("norm", layer.ffn_norm) if layer.ffn is not None else None
+        self.ffn_out_norm = make_part("norm", layer.ffn_out_norm) if layer.ffn is not None else None
+        self.names = tuple(names)
+        self.graph_safe = all(p.graph_safe for p in self._parts())
+
+    def _norms(self):
+        return [(n, p) for n, p in zip(self.names, (self.mixer_norm, self.mixer_out_norm, self.ffn_norm, self.ffn_out_norm))
+                if p is not None]
+
+    def _parts(self):
+        return [self.mixer] + ([self.ffn] if self.ffn is not None else []) + [p for _, p in self._norms()]
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        out: Dict[str, WeightSpec] = {}
+        for name, norm in self._norms():
+            for k, v in norm.weight_specs().items():
+                out[name + k] = v
+        out.update(self.mixer.weight_specs())
+        if self.ffn is not None:
+            out.update(self.ffn.weight_specs())
+        return out
+
+    def load(self, tensors, compute_dtype) -> None:
+        def sub(prefix):
+            return {k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)}
+        for name, norm in self._norms():
+            norm.load(sub(name), compute_dtype)
+        self.mixer.load(tensors, compute_dtype)
+        if self.ffn is not None:
+            self.ffn.load(tensors, compute_dtype)
+
+    def may_capture(self, n_rows: int) -> bool:
+        return all(p.may_capture(n_rows) for p in self._parts())
+
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        return any(p.prefers_eager(n_new, len_before, device) for p in self._parts())
+
+    def entry_norm(self):
+        """The norm that reads the stream first: whoever completes the stream before this block
+        may run it on the way (`Norm.add_to`'s `then`)."""
+        return self.mixer_norm
+
+    def forward(self, ctx, run, x: torch.Tensor, norm_after=None) -> None:
+        ctx.host.pop("stream_copy", None)        # this block writes the stream: a copy of it goes stale
+        ws = ctx.workspace
+        y = ws.get("block_y", tuple(x.shape), ctx.dtype)
+        z = ws.get("block_z", tuple(x.shape), torch.float32)
+        y1 = read_through_norm(ctx, self.mixer_norm, x, y)
+        take_row_factor(ctx, usable=False)       # a norm cut in two by an earlier product is completed here
+        bias = OutputNormBlock._result(ctx, self.mixer, z, run, y1)
+        after = self.ffn_norm if self.ffn is not None else norm_after
+        self.mixer_out_norm.add_to(ctx, z, x, bias=bias, then=None if after is None else (after, y))
+        if self.ffn is None:
+            return
+        y2 = read_through_norm(ctx, self.ffn_norm, x, y)
+        take_row_factor(ctx, usable=False)
+        bias = OutputNormBlock._result(ctx, self.ffn, z, y2)
+        self.ffn_out_norm.add_to(ctx, z, x, bias=bias, then=None if norm_after is None else (norm_after, y))
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "sandwich_norm", SandwichNormBlock)
 register_part("block", "output_norm", OutputNormBlock)

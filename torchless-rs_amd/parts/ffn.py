@@ -1,7 +1,9 @@
 """Gated feed-forward: down( act(gate y) * (up y) ).  With act = silu,
 silu(g) = g / (1 + e^-g), it is SwiGLU (src/model/modules/mlp.rs:23-45,
 src/kernels/mod.rs:546-548 of the reference); `activation` chooses another
-function of the gate (`ops.ACTIVATIONS`: gelu_tanh, the tanh form of gelu).
+function of the gate (`ops.ACTIVATIONS`: gelu_tanh, the tanh form of gelu;
+swish_clamped, g' logistic(alpha g') (u' + shift) on a gate clamped from above and
+an up clamped on both sides, whose constants come in `activation_constants`).
 gate and up are bound under their own names (`names`: the leaf names are
 parameters, and a checkpoint that stores gate|up as one tensor binds that one)
 and laid side by side at load so that one product serves both."""
@@ -26,10 +28,16 @@ class SwiGLU(FeedForward):
     NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", "gate_up": None}
 
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp.",
-                 names: Optional[Dict[str, Optional[str]]] = None, activation: str = "silu"):
+                 names: Optional[Dict[str, Optional[str]]] = None, activation: str = "silu",
+                 activation_constants: Optional[Dict[str, float]] = None):
         if activation not in ops.ACTIVATIONS:
             raise ValueError(f"gated feed-forward: no activation {activation!r}; there are {sorted(ops.ACTIVATIONS)}")
+        need = set(ops.ACTIVATION_CONSTANTS.get(activation, ()))
+        if set(activation_constants or {}) != need:
+            raise ValueError(f"gated feed-forward: {activation!r} takes the constants {sorted(need)}, "
+                             f"got {sorted(activation_constants or {})}")
         self.activation = activation
+        self.constants = dict(activation_constants or {}) or None
         self.H = int(hidden_size)
         self.I = int(intermediate_size)
         self.prefix = prefix
@@ -62,7 +70,7 @@ class SwiGLU(FeedForward):
         # bfloat16 on the matrix cores: gate and up rows interleaved so that the product's
         # epilogue applies silu(gate) * up itself and writes bfloat16
         self.paired = (compute_dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and self.I % 32 == 0
-                       and self.H % 8 == 0)
+                       and self.H % 8 == 0 and self.activation in ops.PAIR_EPILOGUES)
         self.gate_up = Linear(interleave_pairs(g, u) if self.paired else torch.cat([g, u], dim=0))
         self.down = Linear(tensors[p + nm["down"]], tiled=True)
 
@@ -91,7 +99,7 @@ class SwiGLU(FeedForward):
         else:
             gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
             self.gate_up(y, gu)
-            ops.act_mul(gu, h, self.activation)
+            ops.act_mul(gu, h, self.activation, self.constants)
         return h
 
 

@@ -18,16 +18,36 @@ class RMSNorm(Norm):
     graph_safe = True
     takes_pending = True        # adds partial products left in ctx.pending while it reads the stream
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, name: str = "weight"):
+        """`name`: the weight's leaf name behind the norm's prefix ("" where the prefix is the tensor)."""
         self.size = int(size)
         self.eps = float(eps)
+        self.name = name
         self.weight = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((self.size,), init="ones")}
+        return {self.name: WeightSpec((self.size,), init="ones")}
 
     def load(self, tensors, compute_dtype) -> None:
-        self.weight = tensors["weight"].to(torch.float32).contiguous()
+        self.weight = tensors[self.name].to(torch.float32).contiguous()
+
+    def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None, then=None) -> None:
+        """x += norm(z + bias) in one kernel.  `then` = (norm, buffer): the norm that reads the
+        stream next, if it has this form too, runs on the new row in the same kernel and leaves its
+        result in `buffer`; `read_through_norm` of that norm then finds it done."""
+        if bias is not None:
+            z += bias
+        nxt = then[0].rms_form() if then is not None else None
+        if nxt is not None and nxt.size == self.size:
+            ops.rmsnorm_add(z, self.weight, self.eps, x, nxt.weight, nxt.eps, then[1])
+            ctx.prenormed = (then[0], then[1], None)
+        else:
+            ops.rmsnorm_add(z, self.weight, self.eps, x)
+        if out is not None:
+            if out.dtype == torch.float32:
+                out.copy_(x)
+            else:
+                ops.cast_rows(x, out)
 
     def rms_form(self) -> RmsForm:
         return RmsForm(self.weight, self.size, self.eps)
@@ -71,7 +91,7 @@ class LayerNorm(Norm):
             ctx.pending = None
         ops.layernorm(x, self.weight, self.eps, out)
 
-    def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None) -> None:
+    def add_to(self, ctx, z: torch.Tensor, x: torch.Tensor, out=None, bias=None, then=None) -> None:
         ops.layernorm(z, self.weight, self.eps, out, add_to=x, bias=bias)
 
 

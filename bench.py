@@ -69,9 +69,51 @@ def design_configs(z: dict, layers: int, share_from=None):
     return soz, mis
 
 
+def fanitar_config(z: dict, layers: int):
+    """config.json of a Fanitar model with the layer sizes `z`: layers out of latents and differential
+    layers in turn.  The differential layers have half the heads with two maps each and values of two
+    maps' width, so that every projection is as large as the other designs'; the latents are 3/8 and
+    1/8 of the width."""
+    def mixer(i):
+        if i % 2 == 0:
+            m = {"heads": z["heads"], "dim": z["dim"], "vdim": z["dim"], "q_rank": 3 * z["width"] // 8,
+                 "kv_rank": z["width"] // 8, "scale": z["dim"] ** -0.5}
+            if z["window"]:
+                m["mask"] = {"size": z["window"]}
+            return "latent_attention", m
+        return "attention", {"heads": z["heads"] // 2, "kv_heads": z["kv_heads"] // 2, "dim": z["dim"], "vdim": 2 * z["dim"],
+                             "scale": z["dim"] ** -0.5, "diff": 0.5, "rot": {"base": 10000.0, "dims": z["dim"]}}
+    return {"architecture": "Fanitar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 1.0}, "logit_scale": 1.0,
+            "layers": [{"type": mixer(i)[0], "mixer": mixer(i)[1], "mlp": {"kind": "dense", "ff": z["ff"], "limit": 7.0}}
+                       for i in range(layers)]}
+
+
+def fanitar_counts(z: dict, layers: int, B: int, C: int, T: int):
+    """(weight elements of the layers' products, bytes of keys and values that a decode step reads, multiply-adds
+    times two of a prompt's attention) of `fanitar_config(z, layers)`.  The layers out of latents keep keys and
+    values per head (every head its own), the differential ones one key of two maps and one value per KV head;
+    a differential head's two maps are counted with the d channels each that they have."""
+    H, I, nq, nkv, d = z["width"], z["ff"], z["heads"], z["kv_heads"], z["dim"]
+    qr, kvr = 3 * H // 8, H // 8
+    w = kv = att = 0
+    for i in range(layers):
+        w += 3 * I * H
+        if i % 2 == 0:
+            held = min(C, z["window"]) if z["window"] else C
+            w += qr * H + nq * d * qr + kvr * H + 2 * nq * d * kvr + 2 * nq * d * H
+            kv += B * held * nq * 2 * d * 2
+            att += 4 * nq * d * sum(min(p + 1, z["window"] or T) for p in range(T))
+        else:
+            w += 2 * nq * d * H + 2 * nkv * d * H
+            kv += B * C * (nkv // 2) * 4 * d * 2
+            att += (nq // 2) * 2 * (2 * d + 2 * 2 * d) * T * (T + 1) // 2
+    return w, kv, att
+
+
 def bench_designs(args) -> int:
     """Prefill (one prompt of --prefill-tokens in one step) and decode (--batch sequences at --context
-    positions, one token a step through captured graphs) of the two designs at equal layer sizes,
+    positions, one token a step through captured graphs) of the three designs at equal layer sizes,
     random weights, bfloat16.  The bytes a decode step must read (every weight once, the live keys
     and values) over its time is its share of the HBM roofline; a prefill's products and causal
     attention over its time its share of the matrix cores' peak."""
@@ -88,14 +130,15 @@ def bench_designs(args) -> int:
     out = {"metric": "designs_side_by_side", "dtype": "bf16", "data": "synthetic", "layers": L, "batch": B,
            "context": C, "prefill_tokens": T, "steps": args.steps, "warmup": args.warmup, "sizes": {}}
 
-    def measure(cfgd, z, shared_layers=0):
+    def measure(cfgd, z, shared_layers=0, counts=None):
         cfg = config_from_dict(cfgd)
         tensors = random_tensors(model_spec_for(cfg).weight_specs(), seed=5, std=0.02, dtype=torch.bfloat16, device=dev)
         model = model_from_tensors(cfg, tensors, "bfloat16", dev)
         del tensors
         V = z["vocab"]
         held = min(C, z["window"]) if z["window"] else C
-        eng = Engine(model, max_tokens=max(B * (round_up(held) + PAGE), round_up(T) + PAGE), max_slots=max(B, 1),
+        room = C if counts is not None else held          # (a design whose layers differ: some keep every position)
+        eng = Engine(model, max_tokens=max(B * (round_up(room) + PAGE), round_up(T) + PAGE), max_slots=max(B, 1),
                      freeze_gc=False)
         # prefill
         ids = torch.randint(0, V, (T,), generator=gen).tolist()
@@ -132,6 +175,9 @@ def bench_designs(args) -> int:
         w_elems = L * (2 * nq * d * H + 3 * I * H) + own * 2 * nkv * d * H + V * H      # (biases, norms, gates: noise)
         kv_bytes = B * held * 2 * nkv * d * 2 * L           # every layer reads its keys and values, shared or not
         flops = 2 * T * (w_elems - V * H) + 2 * V * H + L * 4 * nq * d * sum(min(p + 1, z["window"] or T) for p in range(T))
+        if counts is not None:
+            w_elems, kv_bytes, att = counts[0] + V * H, counts[1], counts[2]
+            flops = 2 * T * counts[0] + 2 * V * H + att
         return {"prefill_ms": round(pre * 1e3, 3), "prefill_tok_s": round(T / pre),
                 "prefill_frac_of_2.5_pflops": round(flops / pre / 2.5e15, 3),
                 "decode_ms": round(dec * 1e3, 3), "decode_tok_s": round(B / dec),
@@ -140,7 +186,8 @@ def bench_designs(args) -> int:
     for name in [n for n in args.design_sizes.split(",") if n]:
         z = DESIGN_SIZES[name]
         soz, mis = design_configs(z, L)
-        row = {"sozetar": measure(soz, z), "mistral": measure(mis, z)}
+        row = {"fanitar": measure(fanitar_config(z, L), z, counts=fanitar_counts(z, L, B, C, T)),
+               "sozetar": measure(soz, z), "mistral": measure(mis, z)}
         if L > 2:
             row["sozetar_sharing_keys"] = measure(design_configs(z, L, share_from=L // 2 - 1)[0], z, L - L // 2)
         out["sizes"][name] = dict(z, **row)
@@ -171,7 +218,7 @@ def main() -> int:
     ap.add_argument("--only", choices=["prefill", "decode", "pipes", "designs"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling); pipes: whether a "
                          "SIMD's matrix and vector pipes overlap (ops.measure_pipes); designs: prefill and decode of "
-                         "the Sozetar design beside the Mistral design at equal layer sizes (--design-sizes, "
+                         "the Fanitar and Sozetar designs beside the Mistral design at equal layer sizes (--design-sizes, "
                          "--layers, --batch, --context, --prefill-tokens apply)")
     ap.add_argument("--design-sizes", default="2b,7b,12b",
                     help="with --only designs: which layer sizes to run (of %s)" % ",".join(sorted(DESIGN_SIZES)))

@@ -81,13 +81,14 @@ diff_split_kernel(const float* __restrict__ proj, const float* __restrict__ bias
   }
 }
 
-// att[n, 2H, dv]: head 2h is map 1 of head h, 2h + 1 its map 2.  One wave per (row, head).
-template <typename T>
+// att[n, 2H, dv] (TA: the compute type, or float from a kernel that leaves its sums unrounded):
+// head 2h is map 1 of head h, 2h + 1 its map 2.  One wave per (row, head).
+template <typename TA, typename T>
 __global__ void __launch_bounds__(64)
-diff_combine_kernel(const T* __restrict__ att, int H, int dv, float lambda, float eps, float post, T* __restrict__ out) {
+diff_combine_kernel(const TA* __restrict__ att, int H, int dv, float lambda, float eps, float post, T* __restrict__ out) {
   const int n = blockIdx.x / H, h = blockIdx.x % H;
-  const T* a1 = att + ((size_t)n * 2 * H + 2 * h) * dv;
-  const T* a2 = a1 + dv;
+  const TA* a1 = att + ((size_t)n * 2 * H + 2 * h) * dv;
+  const TA* a2 = a1 + dv;
   float o[DIFF_MAX_D / WAVE];
   float ss = 0.f;
 #pragma unroll
@@ -136,8 +137,9 @@ int tl_diff_split(const float* proj, const float* bias, const int* row_pos, cons
   return 0;
 }
 
-int tl_diff_combine(const void* att, int n, int H, int dv, float lambda, float eps, float post, void* out, int dt,
-                    hipStream_t st) {
+int tl_diff_combine(const void* att, int att_dt, int n, int H, int dv, float lambda, float eps, float post, void* out,
+                    int dt, hipStream_t st) {
+  TL_REQUIRE(att_dt == dt || att_dt == DT_F32, "diff_combine: the maps are of the result's type or float");
   TL_REQUIRE(n >= 0 && H > 0 && dv > 0 && dv <= DIFF_MAX_D, "diff_combine: bad sizes n=%d H=%d dv=%d (values up to %d)",
              n, H, dv, DIFF_MAX_D);
   TL_REQUIRE((long long)n * H < 2147483647LL, "diff_combine: too many (row, head) pairs");
@@ -145,9 +147,11 @@ int tl_diff_combine(const void* att, int n, int H, int dv, float lambda, float e
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "diff_combine: unknown dtype code %d", dt);
   if (n == 0) return 0;
   if (dt == DT_F32)
-    diff_combine_kernel<float><<<n * H, 64, 0, st>>>((const float*)att, H, dv, lambda, eps, post, (float*)out);
+    diff_combine_kernel<float, float><<<n * H, 64, 0, st>>>((const float*)att, H, dv, lambda, eps, post, (float*)out);
+  else if (att_dt == DT_F32)
+    diff_combine_kernel<float, bf16><<<n * H, 64, 0, st>>>((const float*)att, H, dv, lambda, eps, post, (bf16*)out);
   else
-    diff_combine_kernel<bf16><<<n * H, 64, 0, st>>>((const bf16*)att, H, dv, lambda, eps, post, (bf16*)out);
+    diff_combine_kernel<bf16, bf16><<<n * H, 64, 0, st>>>((const bf16*)att, H, dv, lambda, eps, post, (bf16*)out);
   TL_LAUNCH_CHECK("diff_combine");
   return 0;
 }

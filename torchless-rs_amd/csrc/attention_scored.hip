@@ -33,13 +33,14 @@ struct ScoreTerms {
 
 // One wave per (row, head): the kernel of the 32-bit path and of every shape that the
 // matrix-core kernels do not take; the reference the faster ones are checked against.
-template <typename T>
+// TO: the type of the result, T or float (for a caller that goes on in float).
+template <typename T, typename TO>
 __global__ void __launch_bounds__(64)
 attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, const T* __restrict__ v_new,
                          const T* __restrict__ pages, const int* __restrict__ table, int table_stride,
                          int ring_pages, const int* __restrict__ row_seq, const int* __restrict__ row_pos,
                          const int* __restrict__ cu_seqlens, const int* __restrict__ n_cached, int nq,
-                         int nkv, int dk, int dv, ScoreTerms terms, T* __restrict__ out) {
+                         int nkv, int dk, int dv, ScoreTerms terms, TO* __restrict__ out) {
   __shared__ float q_s[SC_MAX_D];
   __shared__ float p_s[WAVE];
   __shared__ const T* v_s[WAVE];
@@ -111,11 +112,11 @@ attn_scored_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, c
     }
   }
   const float g = terms.gate ? terms.gate[(size_t)n * nq + h] : 1.f;
-  T* o = out + ((size_t)n * nq + h) * dv;
+  TO* o = out + ((size_t)n * nq + h) * dv;
 #pragma unroll
   for (int i = 0; i < SC_MAX_D / WAVE; ++i) {
     const int dim = lane + WAVE * i;
-    if (dim < dv) o[dim] = from_f32<T>((acc[i] / l) * g);
+    if (dim < dv) o[dim] = from_f32<TO>((acc[i] / l) * g);
   }
 }
 
@@ -340,7 +341,8 @@ int tl_attn_scored_plain(const void* q, const void* k_new, const void* v_new, co
                          const int* table, int table_stride, int ring_pages, const int* row_seq,
                          const int* row_pos, const int* cu_seqlens, const int* n_cached, int n, int nq,
                          int nkv, int dk, int dv, int window, float scale, const float* slopes,
-                         const float* sinks, const float* gate, void* out, hipStream_t st) {
+                         const float* sinks, const float* gate, void* out, int out_dt, hipStream_t st) {
+  TL_REQUIRE(out_dt == dt || out_dt == DT_F32, "scored attention: the result is of the operands' type or float");
   TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "scored attention: bad head counts nq=%d nkv=%d",
              nq, nkv);
   TL_REQUIRE(dk > 0 && dk <= SC_MAX_D && dv > 0 && dv <= SC_MAX_D,
@@ -352,11 +354,15 @@ int tl_attn_scored_plain(const void* q, const void* k_new, const void* v_new, co
   if (n == 0) return 0;
   const ScoreTerms terms{scale, window, slopes, sinks, gate};
   if (dt == DT_F32)
-    attn_scored_plain_kernel<float><<<n * nq, 64, 0, st>>>(
+    attn_scored_plain_kernel<float, float><<<n * nq, 64, 0, st>>>(
         (const float*)q, (const float*)k_new, (const float*)v_new, (const float*)pages, table, table_stride,
         ring_pages, row_seq, row_pos, cu_seqlens, n_cached, nq, nkv, dk, dv, terms, (float*)out);
+  else if (dt == DT_BF16 && out_dt == DT_F32)
+    attn_scored_plain_kernel<bf16, float><<<n * nq, 64, 0, st>>>(
+        (const bf16*)q, (const bf16*)k_new, (const bf16*)v_new, (const bf16*)pages, table, table_stride,
+        ring_pages, row_seq, row_pos, cu_seqlens, n_cached, nq, nkv, dk, dv, terms, (float*)out);
   else if (dt == DT_BF16)
-    attn_scored_plain_kernel<bf16><<<n * nq, 64, 0, st>>>(
+    attn_scored_plain_kernel<bf16, bf16><<<n * nq, 64, 0, st>>>(
         (const bf16*)q, (const bf16*)k_new, (const bf16*)v_new, (const bf16*)pages, table, table_stride,
         ring_pages, row_seq, row_pos, cu_seqlens, n_cached, nq, nkv, dk, dv, terms, (bf16*)out);
   else

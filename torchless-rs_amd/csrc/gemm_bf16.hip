@@ -50,13 +50,28 @@ constexpr int EPI_SILU_PAIR = 2;    // W's rows come in groups of 64 (32 gate ro
                                     // C is bfloat16 [M, N/2] = silu(gate) * up
 constexpr int EPI_GELU_PAIR = 3;    // the same pairs with the tanh form of gelu on the gate:
                                     // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+constexpr int EPI_SWISH_CLAMPED_PAIR = 4;   // the same pairs with g' = min(g, limit), u' = clamp(u, -limit, limit):
+                                            // g' / (1 + exp(-alpha g')) * (u' + shift)
 __host__ __device__ __forceinline__ bool is_pair(int epilogue) {
-  return epilogue == EPI_SILU_PAIR || epilogue == EPI_GELU_PAIR;
+  return epilogue == EPI_SILU_PAIR || epilogue == EPI_GELU_PAIR || epilogue == EPI_SWISH_CLAMPED_PAIR;
 }
-// the gate's function in a paired epilogue, on the float sums
-__device__ __forceinline__ float pair_act(float g, int epilogue) {
-  if (epilogue == EPI_GELU_PAIR) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-  return g / (1.0f + expf(-g));
+// What happens to the product as the kernels take it: the code, and the constants of a paired epilogue
+// whose function has some.  It reads as its code wherever a plain number is asked for.
+struct Epi {
+  int code;
+  float alpha, limit, shift;
+  __host__ __device__ Epi(int c = EPI_STORE, float a = 1.f, float l = 0.f, float s = 0.f) : code(c), alpha(a), limit(l), shift(s) {}
+  __host__ __device__ __forceinline__ operator int() const { return code; }
+};
+// act(gate) * up of a paired epilogue, on the float sums
+__device__ __forceinline__ float pair_value(float g, float u, const Epi& e) {
+  if (e.code == EPI_SWISH_CLAMPED_PAIR) {
+    g = fminf(g, e.limit);
+    u = fminf(fmaxf(u, -e.limit), e.limit);
+    return (g / (1.0f + expf(-e.alpha * g))) * (u + e.shift);
+  }
+  if (e.code == EPI_GELU_PAIR) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+  return (g / (1.0f + expf(-g))) * u;
 }
 
 // An RMSNorm cut in two around a product of at most 16 rows, so that the norm needs no
@@ -143,7 +158,7 @@ tile_weights_kernel(const bf16* __restrict__ W, const int* __restrict__ rows, in
 template <int NT, int MT, int SK_WAVES, bool FULLK, bool TILED = false>      // FULLK: K % 64 == 0, no load needs a guard (and a branch)
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                   int N, int K, int epilogue, NormSplit ns, int rows_per_wg) {
+                   int N, int K, Epi epilogue, NormSplit ns, int rows_per_wg) {
   // rows_per_wg: the channels a workgroup owns, at most 16 NT (0: all 16 NT).  A compute unit streams
   // at a rate of its own, so a product is fastest when every unit has the same share of W: the
   // launcher picks N / units where that is no multiple of 16, and the lanes of an MFMA tile that
@@ -267,7 +282,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
         const int n = (n0 / 2) + jl;
         if (n < NH && m < M) {
           const float g = total(grp * 64 + j, m), u = total(grp * 64 + 32 + j, m);
-          H[(size_t)m * NH + n] = (bf16)(pair_act(g, epilogue) * u);
+          H[(size_t)m * NH + n] = (bf16)pair_value(g, u, epilogue);
         }
       }
     }
@@ -298,7 +313,7 @@ static bool tiles_fit(int N, int K) { return N % 16 == 0 && K % 64 == 0; }
 static int tile_height(int R) { return R > 16 ? R : 16; }
 
 template <int NT, int MT, int SK_WAVES = 8>
-static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
+static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, Epi epilogue,
                          hipStream_t st, NormSplit ns = NormSplit{}, const bf16* Wt = nullptr, int rows_per_wg = 0,
                          int wt_height = 16) {
   const int R = rows_per_wg > 0 ? rows_per_wg : 16 * NT;
@@ -346,7 +361,7 @@ static int balanced_share(int N) {
 
 // the product for at most 16 rows and not many channels, in balanced shares
 static int launch_shares(const bf16* A, const bf16* W, const bf16* Wt, int wt_height, float* C, int M, int N, int K,
-                         int epilogue, hipStream_t st, NormSplit ns, int share) {
+                         Epi epilogue, hipStream_t st, NormSplit ns, int share) {
   if (share <= 16) return launch_skinny<1, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share, wt_height);
   return launch_skinny<2, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share, wt_height);
 }
@@ -366,7 +381,7 @@ constexpr int NRB = 4;                                   // groups of 16 channel
 
 __global__ void __launch_bounds__(256, 2)
 gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
-                 int K, int epilogue, NormSplit ns) {
+                 int K, Epi epilogue, NormSplit ns) {
   extern __shared__ __attribute__((aligned(16))) unsigned char rows_smem[];
   __shared__ float rs[16];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, li = lane % 16, kg = lane / 16;
@@ -438,7 +453,7 @@ gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
       const int j = e % 32, m = e / 32;
       if (m < M) {
         const float g = total(j, m), u = total(32 + j, m);
-        H[(size_t)m * NH + n0 / 2 + j] = (bf16)(pair_act(g, epilogue) * u);
+        H[(size_t)m * NH + n0 / 2 + j] = (bf16)pair_value(g, u, epilogue);
       }
     }
     return;
@@ -454,7 +469,7 @@ gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
 
 static bool rows_fit(int M, int N, int K) { return M <= 16 && N % 64 == 0 && K % ROWS_CHUNK == 0; }
 
-static int launch_rows(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue, hipStream_t st,
+static int launch_rows(const bf16* A, const bf16* W, float* C, int M, int N, int K, Epi epilogue, hipStream_t st,
                        NormSplit ns = NormSplit{}) {
   static bool raised = false;
   if (!raised) {
@@ -637,7 +652,7 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
 template <int MT, int KS, bool FULLK>   // KS: k per step (a multiple of 64), everything of a step is in flight at once;
 __global__ void __launch_bounds__(256)  // FULLK: K % KS == 0, no load needs a guard (and a branch)
 gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                int N, int K, int steps_per_split, int epilogue) {
+                int N, int K, int steps_per_split, Epi epilogue) {
   constexpr int ROWS = MT * 16, LD = KS + 8, SUB = KS / 64;
   __shared__ __attribute__((aligned(16))) bf16 As[ROWS * LD];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, li = lane % 16, kg = lane / 16;
@@ -728,7 +743,7 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
           const int m = 16 * u + 4 * kg + r;
           if (m < M && n < NH) {
             const float g = acc[u][r], up = ex[((wave * MT + u) * 4 + r) * 64 + lane];
-            H[(size_t)m * NH + n] = (bf16)(pair_act(g, epilogue) * up);
+            H[(size_t)m * NH + n] = (bf16)pair_value(g, up, epilogue);
           }
         }
     }
@@ -754,7 +769,7 @@ constexpr int MID_KS = 256;       // k per step up to 64 rows; half of it above,
 constexpr int MID_ROWS = 128;
 
 template <int MT>
-static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
+static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, Epi epilogue,
                       hipStream_t st) {
   constexpr int KS = MT > 4 ? MID_KS / 2 : MID_KS;
   const int steps = (K + KS - 1) / KS, per = (steps + n_split - 1) / n_split;
@@ -789,7 +804,7 @@ template <int N> __device__ __forceinline__ void wait_loads_but() {       // unt
 template <int MT, int WAVES, int KC, int NS>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
-                 int K, int stages_per_split, int epilogue) {
+                 int K, int stages_per_split, Epi epilogue) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char ring_smem[];
   constexpr int ROWB = KC * 2;                              // bytes of a row in a stage
   constexpr int RPI = 1024 / ROWB;                          // rows a load instruction takes
@@ -903,7 +918,7 @@ gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
           const int m = 16 * u + 4 * kg + r;
           if (m < M && n < NH) {
             const float g = acc[u][r], up = ex[(((grp * 2 + wq) * MT + u) * 4 + r) * 64 + lane];
-            H[(size_t)m * NH + n] = (bf16)(pair_act(g, epilogue) * up);
+            H[(size_t)m * NH + n] = (bf16)pair_value(g, up, epilogue);
           }
         }
     }
@@ -926,7 +941,7 @@ gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
 }
 
 template <int MT, int WAVES, int KC>
-static int launch_ring(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
+static int launch_ring(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, Epi epilogue,
                        hipStream_t st) {
   constexpr int STAGE = (MT + WAVES) * 16 * KC * 2;
   constexpr int FIT = (RING_LDS - 1024) / STAGE;
@@ -951,7 +966,7 @@ static int launch_ring(const bf16* A, const bf16* W, float* C, int M, int N, int
 }
 
 template <int WAVES, int KC>
-static int launch_ring_rows(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
+static int launch_ring_rows(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, Epi epilogue,
                             hipStream_t st) {
   if (M <= 32) return launch_ring<2, WAVES, KC>(A, W, C, M, N, K, n_split, epilogue, st);
   if (M <= 64) return launch_ring<4, WAVES, KC>(A, W, C, M, N, K, n_split, epilogue, st);
@@ -963,6 +978,18 @@ static int launch_ring_rows(const bf16* A, const bf16* W, float* C, int M, int N
 
 using namespace tl;
 
+// The constants of EPI_SWISH_CLAMPED_PAIR for the calls that follow on this thread (the kernels get them
+// by value with every launch, so a captured launch keeps the ones it was captured with).
+static thread_local float g_pair_alpha = 1.f, g_pair_limit = 0.f, g_pair_shift = 0.f;
+extern "C" int tl_pair_constants(float alpha, float limit, float shift) {
+  TL_REQUIRE(limit > 0.f, "paired epilogue: the clamp needs a positive limit, got %g", (double)limit);
+  g_pair_alpha = alpha; g_pair_limit = limit; g_pair_shift = shift;
+  return 0;
+}
+static Epi epi_of(int epilogue) {
+  return epilogue == EPI_SWISH_CLAMPED_PAIR ? Epi(epilogue, g_pair_alpha, g_pair_limit, g_pair_shift) : Epi(epilogue);
+}
+
 // epilogue: 0 store float, 1 accumulate into float, 2 silu(gate) * up into bfloat16 [M, N/2]
 // (W's rows in groups of 64: 32 gate rows and their 32 up rows; N a multiple of 64).
 // Wt (or null): the tiled copy of W with tiles of wt_height rows, see tl_gemm_bf16_norm.
@@ -972,7 +999,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, int wt
   TL_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0),
              "gemm_bf16: operands must be 16-byte aligned");
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_bf16: unknown epilogue %d", epilogue);
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 4, "gemm_bf16: unknown epilogue %d", epilogue);
   TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   if (M == 0) return 0;
@@ -981,17 +1008,17 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, int wt
   float* c = (float*)C;
   const bool wide = N >= 16384 || is_pair(epilogue);     // many rows: 64 a workgroup
   if (M <= 16) {
-    if (wide && rows_fit(M, N, K)) return launch_rows(a, w, c, M, N, K, epilogue, st);
-    if (wide && (M > 4 || is_pair(epilogue))) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
-    return launch_shares(a, w, (const bf16*)Wt, wt_height, c, M, N, K, epilogue, st, NormSplit{}, balanced_share(N));
+    if (wide && rows_fit(M, N, K)) return launch_rows(a, w, c, M, N, K, epi_of(epilogue), st);
+    if (wide && (M > 4 || is_pair(epilogue))) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    return launch_shares(a, w, (const bf16*)Wt, wt_height, c, M, N, K, epi_of(epilogue), st, NormSplit{}, balanced_share(N));
   }
   if (M <= 32) {
-    if (wide) return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
-    return launch_skinny<2, 2, 8>(a, w, c, M, N, K, epilogue, st);
+    if (wide) return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    return launch_skinny<2, 2, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
   }
   if (M <= 64) {
-    if (wide) return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epilogue, st);
-    return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epilogue, st);
+    if (wide) return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
   }
   TL_REQUIRE(false, "gemm_bf16: %d rows; this entry point serves at most 64 (tl_gemm_mid_bf16 takes up to 128, "
              "the BLAS library more)", M);
@@ -1010,28 +1037,28 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
   if (variant == 2) {
     TL_REQUIRE(rows_fit(M, N, K), "gemm_rows: M=%d N=%d K=%d (at most 16 rows, N a multiple of 64, K of %d)", M, N,
                K, ROWS_CHUNK);
-    return launch_rows(a, w, c, M, N, K, epilogue, st);
+    return launch_rows(a, w, c, M, N, K, epi_of(epilogue), st);
   }
   if (variant > 1000 && variant <= 1032) {
     TL_REQUIRE(M <= 16 && !is_pair(epilogue), "gemm_skinny: variant %d takes at most 16 rows and no pairs", variant);
     const int R = variant - 1000;
-    if (R <= 16) return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);
-    return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);
+    if (R <= 16) return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epi_of(epilogue), st, NormSplit{}, nullptr, R);
+    return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epi_of(epilogue), st, NormSplit{}, nullptr, R);
   }
   const int mt = (variant / 10) % 10;
   TL_REQUIRE(M <= 16 * mt, "gemm_skinny: variant %d takes at most %d rows, not %d", variant, 16 * mt, M);
   TL_REQUIRE(!is_pair(epilogue) || variant / 100 == 4, "gemm_skinny: the paired epilogue needs 64 rows "
              "a workgroup (variant 4xx)");
   switch (variant) {
-    case 112: return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st);
-    case 111: return launch_skinny<1, 1, 4>(a, w, c, M, N, K, epilogue, st);
-    case 212: return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epilogue, st);
-    case 411: return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
-    case 222: return launch_skinny<2, 2, 8>(a, w, c, M, N, K, epilogue, st);
-    case 421: return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
-    case 242: return launch_skinny<2, 4, 8>(a, w, c, M, N, K, epilogue, st);
-    case 441: return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epilogue, st);
-    case 142: return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epilogue, st);
+    case 112: return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 111: return launch_skinny<1, 1, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 212: return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 411: return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 222: return launch_skinny<2, 2, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 421: return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 242: return launch_skinny<2, 4, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 441: return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epi_of(epilogue), st);
+    case 142: return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epi_of(epilogue), st);
   }
   TL_REQUIRE(false, "gemm_bf16: unknown variant %d", variant);
 }
@@ -1051,21 +1078,21 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
   TL_REQUIRE(n_split >= 1 && n_split <= (K + MID_KS - 1) / MID_KS && n_split <= 65535,
              "gemm_mid: %d splits do not fit K=%d (one step of %d at least each)", n_split, K, MID_KS);
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 3 && (n_split == 1 || epilogue == EPI_STORE),
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 4 && (n_split == 1 || epilogue == EPI_STORE),
              "gemm_mid: epilogue %d cannot go with %d splits", epilogue, n_split);
   TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_mid: the paired epilogue needs N=%d to be a "
              "multiple of 64", N);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   float* c = (float*)C;
-  if (M <= 16) return launch_mid<1>(a, w, c, M, N, K, n_split, epilogue, st);
-  if (M <= 32) return launch_mid<2>(a, w, c, M, N, K, n_split, epilogue, st);
-  if (M <= 48) return launch_mid<3>(a, w, c, M, N, K, n_split, epilogue, st);
-  if (M <= 64) return launch_mid<4>(a, w, c, M, N, K, n_split, epilogue, st);
-  if (M <= 80) return launch_mid<5>(a, w, c, M, N, K, n_split, epilogue, st);
-  if (M <= 96) return launch_mid<6>(a, w, c, M, N, K, n_split, epilogue, st);
-  if (M <= 112) return launch_mid<7>(a, w, c, M, N, K, n_split, epilogue, st);
-  return launch_mid<8>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 16) return launch_mid<1>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  if (M <= 32) return launch_mid<2>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  if (M <= 48) return launch_mid<3>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  if (M <= 64) return launch_mid<4>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  if (M <= 80) return launch_mid<5>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  if (M <= 96) return launch_mid<6>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  if (M <= 112) return launch_mid<7>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
+  return launch_mid<8>(a, w, c, M, N, K, n_split, epi_of(epilogue), st);
 }
 
 // The same product through the ring kernel (see gemm_ring_kernel): K a multiple of 128.  waves: the waves of a
@@ -1079,7 +1106,7 @@ extern "C" int tl_gemm_ring_bf16(const void* A, const void* W, void* C, int M, i
   TL_REQUIRE(kc == 64 || kc == 128, "gemm_ring: a stage of %d k (64 or 128)", kc);
   TL_REQUIRE(n_split >= 1 && n_split <= K / kc && n_split <= 65535,
              "gemm_ring: %d splits do not fit K=%d (one stage of %d at least each)", n_split, K, kc);
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 3 && (n_split == 1 || epilogue == EPI_STORE),
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 4 && (n_split == 1 || epilogue == EPI_STORE),
              "gemm_ring: epilogue %d cannot go with %d splits", epilogue, n_split);
   TL_REQUIRE(!is_pair(epilogue) || (N % 64 == 0 && waves % 4 == 0), "gemm_ring: the paired epilogue needs N=%d "
              "to be a multiple of 64 and whole groups of four waves (%d)", N, waves);
@@ -1088,8 +1115,8 @@ extern "C" int tl_gemm_ring_bf16(const void* A, const void* W, void* C, int M, i
   float* c = (float*)C;
 #define TL_RING(WV)                                                                                     \
   if (waves == WV)                                                                                      \
-    return kc == 64 ? launch_ring_rows<WV, 64>(a, w, c, M, N, K, n_split, epilogue, st)                 \
-                    : launch_ring_rows<WV, 128>(a, w, c, M, N, K, n_split, epilogue, st)
+    return kc == 64 ? launch_ring_rows<WV, 64>(a, w, c, M, N, K, n_split, epi_of(epilogue), st)                 \
+                    : launch_ring_rows<WV, 128>(a, w, c, M, N, K, n_split, epi_of(epilogue), st)
   TL_RING(4);
   TL_RING(7);
   TL_RING(8);
@@ -1167,7 +1194,7 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, i
   TL_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16_norm: bad sizes M=%d N=%d K=%d (at most "
              "16 rows, K a multiple of 8)", M, N, K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_bf16_norm: operands must be 16-byte aligned");
-  TL_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_bf16_norm: unknown epilogue %d", epilogue);
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 4, "gemm_bf16_norm: unknown epilogue %d", epilogue);
   TL_REQUIRE(!is_pair(epilogue) || N % 64 == 0, "gemm_bf16_norm: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
   TL_REQUIRE(ssq_in == nullptr || n_part > 0, "gemm_bf16_norm: %d partial sums of squares", n_part);
@@ -1186,10 +1213,10 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, i
   NormSplit ns{};
   ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
   ns.norm_w = norm_w; ns.xt = (bf16*)xt; ns.ssq_out = ssq_out;
-  if (rows) return launch_rows((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
-  if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
+  if (rows) return launch_rows((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epi_of(epilogue), st, ns);
+  if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epi_of(epilogue), st, ns);
   TL_REQUIRE((uintptr_t)Wt % 16 == 0, "gemm_bf16_norm: operands must be 16-byte aligned");
-  return launch_shares((const bf16*)A, (const bf16*)W, (const bf16*)Wt, wt_height, (float*)C, M, N, K, epilogue, st, ns,
+  return launch_shares((const bf16*)A, (const bf16*)W, (const bf16*)Wt, wt_height, (float*)C, M, N, K, epi_of(epilogue), st, ns,
                        share);
 }
 

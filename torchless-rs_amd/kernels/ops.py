@@ -424,7 +424,7 @@ def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pag
     """Attention of every row over its sequence's cached keys (j < n_cached) and this step's
     (k_new [n, nkv, dk], v_new [n, nkv, dv]; None when everything is in the pages), causal, with
     the terms of `ScoreTerms`; `gate` (float32 [n, nq] or None) multiplies each head's output.
-    One wave per (row, head), float32 sums."""
+    One wave per (row, head), float32 sums; `out` may be float32 whatever the operands are."""
     n, nq, dk = q.shape
     B = n_cached.shape[0]
     _req(q, "attn_scored.q", pages.dtype)
@@ -437,7 +437,7 @@ def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pag
     _req(row_pos, "attn_scored.row_pos", torch.int32, (n,))
     _req(cu_seqlens, "attn_scored.cu_seqlens", torch.int32, (B + 1,))
     _req(n_cached, "attn_scored.n_cached", torch.int32, (B,))
-    _req(out, "attn_scored.out", pages.dtype, (n, nq, dv))
+    _req(out, "attn_scored.out", torch.float32 if out.dtype == torch.float32 else pages.dtype, (n, nq, dv))
     if terms.slopes is not None:
         _req(terms.slopes, "attn_scored.slopes", torch.float32, (nq,))
     if terms.sinks is not None:
@@ -450,7 +450,7 @@ def attn_scored_plain(q, k_new, v_new, pages, nkv: int, dv: int, table, ring_pag
                                       table.shape[1], ring_pages, _p(row_seq), _p(row_pos), _p(cu_seqlens),
                                       _p(n_cached), n, nq, nkv, dk, dv, int(terms.window or 0),
                                       ctypes.c_float(terms.scale), _p(terms.slopes), _p(terms.sinks), _p(gate),
-                                      _p(out), _stream()))
+                                      _p(out), _code(out.dtype), _stream()))
 
 
 def scored_on_matrix_cores(dtype: torch.dtype, dk: int, dv: int) -> bool:
@@ -652,15 +652,15 @@ def diff_split(proj: torch.Tensor, bias, row_pos, rotation, H: int, G: int, d: i
 
 
 def diff_combine(att: torch.Tensor, lam: float, eps: float, post: float, out: torch.Tensor) -> None:
-    """att [n, 2*H, dv] (heads 2h and 2h + 1: the two maps of head h) -> out [n, H, dv]:
-    o = a1 - lam * a2, then o / sqrt(mean(o^2) + eps) * post, in float32."""
+    """att [n, 2*H, dv] (heads 2h and 2h + 1: the two maps of head h; of out's dtype, or float32) ->
+    out [n, H, dv]: o = a1 - lam * a2, then o / sqrt(mean(o^2) + eps) * post, in float32."""
     n, H2, dv = att.shape
     _req(att, "diff_combine.att")
     if H2 % 2:
         raise KernelError(f"diff_combine: {H2} maps are not pairs")
-    _req(out, "diff_combine.out", att.dtype, (n, H2 // 2, dv))
-    _check(lib().tl_diff_combine(_p(att), n, H2 // 2, dv, ctypes.c_float(lam), ctypes.c_float(eps), ctypes.c_float(post),
-                                 _p(out), _code(att.dtype), _stream()))
+    _req(out, "diff_combine.out", None, (n, H2 // 2, dv))
+    _check(lib().tl_diff_combine(_p(att), _code(att.dtype), n, H2 // 2, dv, ctypes.c_float(lam), ctypes.c_float(eps),
+                                 ctypes.c_float(post), _p(out), _code(out.dtype), _stream()))
 
 
 def take_tokens(src: torch.Tensor, idx: torch.Tensor, vocab: int, tokens: torch.Tensor) -> None:
@@ -708,14 +708,22 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, s
 EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR, EPI_GELU_PAIR = 0, 1, 2, 3
 
 
-PAIR_EPILOGUES = ("silu", "gelu_tanh")       # the gate functions that the products' paired epilogue knows
+EPI_SWISH_CLAMPED_PAIR = 4
+PAIR_EPILOGUES = {"silu": EPI_SILU_PAIR, "gelu_tanh": EPI_GELU_PAIR, "swish_clamped": EPI_SWISH_CLAMPED_PAIR}
 
 
-def _pair_epilogue(pair_act: str) -> int:
-    """The code of the paired epilogue act(gate) * up for the gate's function `pair_act`."""
+def _pair_epilogue(pair_act, constants=None) -> int:
+    """The code of the paired epilogue act(gate) * up for the gate's function `pair_act`: a name of
+    `PAIR_EPILOGUES`, or (name, constants) for a function that has some.  The constants are handed to the
+    library for the launches that follow on this thread (each launch carries them by value)."""
+    if isinstance(pair_act, tuple):
+        pair_act, constants = pair_act
     if pair_act not in PAIR_EPILOGUES:
         raise KernelError(f"paired epilogue: no function {pair_act!r}; there are {sorted(PAIR_EPILOGUES)}")
-    return EPI_GELU_PAIR if pair_act == "gelu_tanh" else EPI_SILU_PAIR
+    k = _act_constants(pair_act, constants)
+    if pair_act in ACTIVATION_CONSTANTS:
+        _check(lib().tl_pair_constants(*k))
+    return PAIR_EPILOGUES[pair_act]
 
 
 def tiles_fit(N: int, K: int) -> bool:

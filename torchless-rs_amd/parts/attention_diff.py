@@ -17,7 +17,9 @@ of 2d channels with its own channels in half m and zeros in the other half, so t
 product with the key is q_m . k_m exactly, the two maps of a head are two heads of the same
 group, and both read the same values once.  (The price is twice the multiplications in the
 score product; the value product and all memory traffic are what two maps need.)
-lambda is worked out once at load, in float32; the difference and its norm are float32.
+lambda is worked out once at load, in float32; the difference and its norm are float32 (of maps
+that the matrix-core kernels have rounded to bfloat16, or of the unrounded maps where the kernel that
+sums in float runs: head sizes the matrix cores do not take, and the 32-bit path).
 """
 from __future__ import annotations
 
@@ -108,7 +110,9 @@ class DifferentialAttentionMixer(Mixer):
         self.proj(y, proj)
         rotation = self.position.rotation(y.device) or ops.NO_ROTATION
         q = ws.get("diff_q", (n, 2 * H, 2 * d), ctx.dtype)
-        maps = ws.get("diff_maps", (n, 2 * H, dv), ctx.dtype)
+        # where the kernel that keeps its sums in float runs, the two maps stay unrounded until their difference
+        cores = ops.scored_on_matrix_cores(ctx.dtype, 2 * d, dv)
+        maps = ws.get("diff_maps", (n, 2 * H, dv), ctx.dtype if cores else torch.float32)
         if ctx.all_single:      # one token a sequence: k and v go straight into the pages
             group = run.kv_group
             ops.diff_split(proj, self.proj_bias, ctx.row_pos, rotation, H, G, d, dv, q, None, None,

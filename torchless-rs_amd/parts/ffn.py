@@ -38,6 +38,7 @@ class SwiGLU(FeedForward):
                              f"got {sorted(activation_constants or {})}")
         self.activation = activation
         self.constants = dict(activation_constants or {}) or None
+        self.pair = (activation, self.constants) if self.constants else activation     # as the products' epilogue takes it
         self.H = int(hidden_size)
         self.I = int(intermediate_size)
         self.prefix = prefix
@@ -86,16 +87,16 @@ class SwiGLU(FeedForward):
         h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
         factor = take_row_factor(ctx, usable=self.paired and ops.norm_split_ok(y, self.gate_up.weight))
         if factor is not None:
-            ops.gemm_bf16_norm(y, self.gate_up.weight, h, silu_pair=True, factor=factor, pair_act=self.activation)
+            ops.gemm_bf16_norm(y, self.gate_up.weight, h, silu_pair=True, factor=factor, pair_act=self.pair)
         elif self.paired and self.gate_up.mid(y):
-            ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True, pair_act=self.activation)
+            ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True, pair_act=self.pair)
         elif self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
             if n > ops.LIBRARY_ROWS:
                 gu = ctx.workspace.get("ffn_gu16", (n, 2 * self.I), torch.bfloat16)
                 ops.gemm_library(y, self.gate_up.weight, gu)
-                ops.silu_mul_pairs(gu, h, self.activation)
+                ops.silu_mul_pairs(gu, h, self.activation, self.constants)
             else:
-                ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True, pair_act=self.activation)
+                ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True, pair_act=self.pair)
         else:
             gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
             self.gate_up(y, gu)

@@ -186,9 +186,15 @@ def bench_designs(args) -> int:
     for name in [n for n in args.design_sizes.split(",") if n]:
         z = DESIGN_SIZES[name]
         soz, mis = design_configs(z, L)
-        row = {"fanitar": measure(fanitar_config(z, L), z, counts=fanitar_counts(z, L, B, C, T)),
-               "sozetar": measure(soz, z), "mistral": measure(mis, z)}
-        if L > 2:
+        which = [n for n in args.design_names.split(",") if n]
+        row = {}
+        if "fanitar" in which:
+            row["fanitar"] = measure(fanitar_config(z, L), z, counts=fanitar_counts(z, L, B, C, T))
+        if "sozetar" in which:
+            row["sozetar"] = measure(soz, z)
+        if "mistral" in which:
+            row["mistral"] = measure(mis, z)
+        if L > 2 and "sozetar" in which:
             row["sozetar_sharing_keys"] = measure(design_configs(z, L, share_from=L // 2 - 1)[0], z, L - L // 2)
         out["sizes"][name] = dict(z, **row)
         print(f"[bench] {name}: {json.dumps(row)}", file=sys.stderr, flush=True)
@@ -220,6 +226,8 @@ def main() -> int:
                          "SIMD's matrix and vector pipes overlap (ops.measure_pipes); designs: prefill and decode of "
                          "the Fanitar and Sozetar designs beside the Mistral design at equal layer sizes (--design-sizes, "
                          "--layers, --batch, --context, --prefill-tokens apply)")
+    ap.add_argument("--design-names", default="fanitar,sozetar,mistral",
+                    help="with --only designs: which designs to run")
     ap.add_argument("--design-sizes", default="2b,7b,12b",
                     help="with --only designs: which layer sizes to run (of %s)" % ",".join(sorted(DESIGN_SIZES)))
     args = ap.parse_args()

@@ -19,19 +19,25 @@ namespace tl {
 
 constexpr int DIFF_MAX_D = 256;
 
-// blockIdx.y: 0 q, 1 k, 2 v
+// A workgroup takes SPLIT_CHUNK consecutive outputs of a row's [q (as laid out: 2 * Q) | k | v]: few rows
+// (single-token steps) then still spread over many workgroups.
+constexpr int SPLIT_CHUNK = 1024;
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 diff_split_kernel(const float* __restrict__ proj, const float* __restrict__ bias, const int* __restrict__ row_pos,
                   Rotation rot, int H, int G, int d, int dv, T* __restrict__ q, T* __restrict__ k, T* __restrict__ v,
                   const int* __restrict__ table, int table_stride, int ring_pages, T* __restrict__ pages) {
   __shared__ float cs[DIFF_MAX_D / 2], sn[DIFF_MAX_D / 2];
-  const int n = blockIdx.x, section = blockIdx.y;
+  const int n = blockIdx.x;
   const int Q = 2 * H * d, K = 2 * G * d, V = G * dv;
+  const int total = 2 * Q + K + V;
+  const int e0 = blockIdx.y * SPLIT_CHUNK;
+  const int e1 = min(total, e0 + SPLIT_CHUNK);
   const float* row = proj + (size_t)n * (Q + K + V);
   const int pos = row_pos[n];
   const int half = rot.rotary_dim / 2;
-  if (section < 2) {
+  if (e0 < 2 * Q + K) {           // some of this chunk is rotated
     for (int i = threadIdx.x; i < half; i += 256) sincosf((float)pos * rot.inv_freq[i], &sn[i], &cs[i]);
     __syncthreads();
   }
@@ -47,16 +53,6 @@ diff_split_kernel(const float* __restrict__ proj, const float* __restrict__ bias
     rotate_pair(at(base + c - half), at(base + c), cs[c - half], sn[c - half], ra, rb);
     return rb;
   };
-  if (section == 0) {
-    // map u = 2h + m becomes the head u of 2d channels, its own channels in half m
-    T* qr = q + (size_t)n * 2 * Q;
-    for (int i = threadIdx.x; i < 2 * Q; i += 256) {
-      const int u = i / (2 * d), c = i % (2 * d), m = u % 2;
-      const bool own = (c / d) == m;
-      qr[i] = from_f32<T>(own ? rotated(u * d, c % d) : 0.f);
-    }
-    return;
-  }
   T* kd = nullptr;
   T* vd = nullptr;
   int r = 0;
@@ -66,18 +62,23 @@ diff_split_kernel(const float* __restrict__ proj, const float* __restrict__ bias
     vd = kd + (size_t)G * PAGE * 2 * d;
     r = pos % PAGE;
   }
-  if (section == 1) {
-    for (int i = threadIdx.x; i < K; i += 256) {
+  for (int e = e0 + threadIdx.x; e < e1; e += 256) {
+    if (e < 2 * Q) {
+      // map u = 2h + m becomes the head u of 2d channels, its own channels in half m
+      const int u = e / (2 * d), c = e % (2 * d), m = u % 2;
+      const bool own = (c / d) == m;
+      q[(size_t)n * 2 * Q + e] = from_f32<T>(own ? rotated(u * d, c % d) : 0.f);
+    } else if (e < 2 * Q + K) {
+      const int i = e - 2 * Q;
       const T t = from_f32<T>(rotated(Q + (i / d) * d, i % d));
       if (pages) kd[((size_t)(i / (2 * d)) * PAGE + r) * 2 * d + i % (2 * d)] = t;
       else k[(size_t)n * K + i] = t;
+    } else {
+      const int i = e - 2 * Q - K;
+      const T t = from_f32<T>(at(Q + K + i));
+      if (pages) vd[(size_t)i * PAGE + r] = t;
+      else v[(size_t)n * V + i] = t;
     }
-    return;
-  }
-  for (int i = threadIdx.x; i < V; i += 256) {
-    const T t = from_f32<T>(at(Q + K + i));
-    if (pages) vd[(size_t)i * PAGE + r] = t;
-    else v[(size_t)n * V + i] = t;
   }
 }
 
@@ -126,7 +127,7 @@ int tl_diff_split(const float* proj, const float* bias, const int* row_pos, cons
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "diff_split: unknown dtype code %d", dt);
   if (n == 0) return 0;
   const Rotation rot{inv_freq, rotary_dim, 0};
-  const dim3 grid(n, 3);
+  const dim3 grid(n, (4 * H * d + 2 * G * d + G * dv + SPLIT_CHUNK - 1) / SPLIT_CHUNK);
   if (dt == DT_F32)
     diff_split_kernel<float><<<grid, 256, 0, st>>>(proj, bias, row_pos, rot, H, G, d, dv, (float*)q, (float*)k, (float*)v,
                                                    table, table_stride, ring_pages, (float*)pages);

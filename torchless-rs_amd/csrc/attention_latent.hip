@@ -42,19 +42,19 @@ latent_norms_kernel(const float* __restrict__ proj, int na, int nb, int ng, cons
 // qf[n, nq*dk] (row stride q_stride), kf[n, nkv*dk] and vf[n, nkv*dv] (row stride kv_stride each, so
 // that k and v may be the two halves of one product) in float -> q, and k and v as rows or
 // (pages != null: row n is sequence n) into the page of the row's position, values transposed.
-// blockIdx.y: 0 q, 1 k, 2 v.
+// A workgroup takes HEADS_CHUNK consecutive outputs of a row's [q | k | v].
+constexpr int HEADS_CHUNK = 1024;
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 split_heads_kernel(const float* __restrict__ qf, int q_stride, const float* __restrict__ kf,
                    const float* __restrict__ vf, int kv_stride, const int* __restrict__ row_pos, int nq, int nkv,
                    int dk, int dv, T* __restrict__ q, T* __restrict__ k, T* __restrict__ v,
                    const int* __restrict__ table, int table_stride, int ring_pages, T* __restrict__ pages) {
-  const int n = blockIdx.x, section = blockIdx.y;
-  if (section == 0) {
-    const int Q = nq * dk;
-    for (int i = threadIdx.x; i < Q; i += 256) q[(size_t)n * Q + i] = from_f32<T>(qf[(size_t)n * q_stride + i]);
-    return;
-  }
+  const int n = blockIdx.x;
+  const int Q = nq * dk, K = nkv * dk, V = nkv * dv;
+  const int e0 = blockIdx.y * HEADS_CHUNK;
+  const int e1 = min(Q + K + V, e0 + HEADS_CHUNK);
   T* kd = nullptr;
   T* vd = nullptr;
   int r = 0;
@@ -65,20 +65,20 @@ split_heads_kernel(const float* __restrict__ qf, int q_stride, const float* __re
     vd = kd + (size_t)nkv * PAGE * dk;
     r = pos % PAGE;
   }
-  if (section == 1) {
-    const int K = nkv * dk;
-    for (int i = threadIdx.x; i < K; i += 256) {
+  for (int e = e0 + threadIdx.x; e < e1; e += 256) {
+    if (e < Q) {
+      q[(size_t)n * Q + e] = from_f32<T>(qf[(size_t)n * q_stride + e]);
+    } else if (e < Q + K) {
+      const int i = e - Q;
       const T t = from_f32<T>(kf[(size_t)n * kv_stride + i]);
       if (pages) kd[((size_t)(i / dk) * PAGE + r) * dk + i % dk] = t;
       else k[(size_t)n * K + i] = t;
+    } else {
+      const int i = e - Q - K;
+      const T t = from_f32<T>(vf[(size_t)n * kv_stride + i]);
+      if (pages) vd[(size_t)i * PAGE + r] = t;          // [kv head][dv][row]: channel i of the row is line i
+      else v[(size_t)n * V + i] = t;
     }
-    return;
-  }
-  const int V = nkv * dv;
-  for (int i = threadIdx.x; i < V; i += 256) {
-    const T t = from_f32<T>(vf[(size_t)n * kv_stride + i]);
-    if (pages) vd[(size_t)i * PAGE + r] = t;          // [kv head][dv][row]: channel i of the row is line i
-    else v[(size_t)n * V + i] = t;
   }
 }
 
@@ -120,7 +120,7 @@ int tl_split_heads(const float* qf, int q_stride, const float* kf, const float* 
              "split_heads: pages without a page table");
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "split_heads: unknown dtype code %d", dt);
   if (n == 0) return 0;
-  const dim3 grid(n, 3);
+  const dim3 grid(n, (nq * dk + nkv * (dk + dv) + HEADS_CHUNK - 1) / HEADS_CHUNK);
   if (dt == DT_F32)
     split_heads_kernel<float><<<grid, 256, 0, st>>>(qf, q_stride, kf, vf, kv_stride, row_pos, nq, nkv, dk, dv, (float*)q,
                                                     (float*)k, (float*)v, table, table_stride, ring_pages, (float*)pages);

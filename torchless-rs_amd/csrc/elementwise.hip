@@ -616,6 +616,63 @@ rmsnorm_add_kernel(const float* __restrict__ z, const float* __restrict__ w, flo
   for (int i = threadIdx.x; i < H; i += 256) o[i] = from_f32<TO>((xr[i] / rms2) * w_next[i]);
 }
 
+// The same with the rows held in registers: z, x and both weights are read once, all loads issued
+// before the first sum.  H % 4 == 0, H <= 1024 * IT.
+template <typename TO, int IT>
+__global__ void __launch_bounds__(256)
+rmsnorm_add_reg_kernel(const float* __restrict__ z, const float* __restrict__ w, float eps, float* __restrict__ x,
+                       const float* __restrict__ w_next, float eps_next, TO* __restrict__ out, int H) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x;
+  const float4* zr = reinterpret_cast<const float4*>(z + (size_t)n * H);
+  float4* xr = reinterpret_cast<float4*>(x + (size_t)n * H);
+  const float4* wr = reinterpret_cast<const float4*>(w);
+  const float4* wn = reinterpret_cast<const float4*>(w_next);
+  const int nv = H / 4;
+  float4 a[IT], v[IT], g[IT], g2[IT];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      a[i] = zr[c];
+      v[i] = xr[c];
+      g[i] = wr[c];
+      if (w_next) g2[i] = wn[c];
+      ss += a[i].x * a[i].x + a[i].y * a[i].y + a[i].z * a[i].z + a[i].w * a[i].w;
+    }
+  }
+  ss = block_sum<256>(ss, sh);
+  const float rms = sqrtf(ss / (float)H + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      v[i].x += (a[i].x / rms) * g[i].x;
+      v[i].y += (a[i].y / rms) * g[i].y;
+      v[i].z += (a[i].z / rms) * g[i].z;
+      v[i].w += (a[i].w / rms) * g[i].w;
+      xr[c] = v[i];
+      s2 += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+  }
+  if (w_next == nullptr) return;
+  s2 = block_sum<256>(s2, sh);
+  const float rms2 = sqrtf(s2 / (float)H + eps_next);
+  TO* o = out + (size_t)n * H;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      o[4 * c + 0] = from_f32<TO>((v[i].x / rms2) * g2[i].x);
+      o[4 * c + 1] = from_f32<TO>((v[i].y / rms2) * g2[i].y);
+      o[4 * c + 2] = from_f32<TO>((v[i].z / rms2) * g2[i].z);
+      o[4 * c + 3] = from_f32<TO>((v[i].w / rms2) * g2[i].w);
+    }
+  }
+}
+
 // x[n, :] += extra[n, :] (may be null) + vec[:]: what a pass over a run of layers adds at its start
 __global__ void stream_entry_kernel(float* __restrict__ x, const float* __restrict__ extra,
                                     const float* __restrict__ vec, int H, size_t total) {
@@ -1006,10 +1063,23 @@ int tl_rmsnorm_add(const float* z, const float* w, float eps, float* x, const fl
   TL_REQUIRE(w_next == nullptr || (out != nullptr && (out_dt == DT_F32 || out_dt == DT_BF16)),
              "rmsnorm_add: the norm that follows needs a buffer of a known type");
   if (n == 0) return 0;
-  if (w_next == nullptr || out_dt == DT_F32)
+  const bool f32 = w_next == nullptr || out_dt == DT_F32;
+  const bool vec = H % 4 == 0 && H <= 8192 && ((uintptr_t)z % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+                   ((uintptr_t)x % 16 == 0) && ((uintptr_t)w_next % 16 == 0);
+#define TL_RMSA(IT)                                                                                                  \
+  do {                                                                                                               \
+    if (f32) rmsnorm_add_reg_kernel<float, IT><<<n, 256, 0, st>>>(z, w, eps, x, w_next, eps_next, (float*)out, H);   \
+    else rmsnorm_add_reg_kernel<bf16, IT><<<n, 256, 0, st>>>(z, w, eps, x, w_next, eps_next, (bf16*)out, H);         \
+  } while (0)
+  if (vec && H <= 1024) TL_RMSA(1);
+  else if (vec && H <= 2048) TL_RMSA(2);
+  else if (vec && H <= 4096) TL_RMSA(4);
+  else if (vec) TL_RMSA(8);
+  else if (f32)
     rmsnorm_add_kernel<float><<<n, 256, 0, st>>>(z, w, eps, x, w_next, eps_next, (float*)out, H);
   else
     rmsnorm_add_kernel<bf16><<<n, 256, 0, st>>>(z, w, eps, x, w_next, eps_next, (bf16*)out, H);
+#undef TL_RMSA
   TL_LAUNCH_CHECK("rmsnorm_add");
   return 0;
 }

@@ -539,6 +539,44 @@ def test_the_right_parts_and_caches_are_chosen(zoo):
     assert eng.runs[0].kv_group.ring_pages == 1 and eng.runs[1].kv_group.request.head_dim == 16
 
 
+def test_which_attention_kernels_run(zoo, monkeypatch):
+    """bfloat16 with head sizes the matrix cores take: the layers out of latents run the kernels with
+    terms (their sink), the differential layers the kernels without, none the one that sums in float;
+    a step of at most 16 rows applies the clamped gate in the product's epilogue, not in a kernel of its own."""
+    from torchless_rs_amd.engine import SeqInput
+    from torchless_rs_amd.kernels import ops
+    eng, z = engine_for(zoo, "cores", "bfloat16"), zoo["cores"]
+    calls = {"plain": 0, "terms": 0, "bare": 0, "act": 0}
+    real_terms, real_bare = ops.attention_scored, ops.attention
+
+    def no_plain(*a, **k):
+        calls["plain"] += 1
+        raise AssertionError("the float kernel ran")
+
+    def terms(*a, **k):
+        calls["terms"] += 1
+        return real_terms(*a, **k)
+
+    def bare(*a, **k):
+        calls["bare"] += 1
+        return real_bare(*a, **k)
+
+    def act(*a, **k):
+        calls["act"] += 1
+        raise AssertionError("the gate ran in a kernel of its own")
+
+    monkeypatch.setattr(ops, "attn_scored_plain", no_plain)
+    monkeypatch.setattr(ops, "attention_scored", terms)
+    monkeypatch.setattr(ops, "attention", bare)
+    monkeypatch.setattr(ops, "act_mul", act)
+    s = eng.alloc()
+    eng.step([SeqInput(s, z["prompts"][2][:100], [99])])
+    eng.step([SeqInput(s, z["prompts"][2][100:101], [0])])
+    eng.free(s)
+    # five runs a step (two passes over the first two layers, then the third): three out of latents, two differential
+    assert calls == {"plain": 0, "terms": 6, "bare": 4, "act": 0}
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_each_request_alone_and_whole(zoo, name, dtype):

@@ -27,13 +27,13 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 diff_split_kernel(const float* __restrict__ proj, const float* __restrict__ bias, const int* __restrict__ row_pos,
                   Rotation rot, int H, int G, int d, int dv, T* __restrict__ q, T* __restrict__ k, T* __restrict__ v,
-                  const int* __restrict__ table, int table_stride, int ring_pages, T* __restrict__ pages) {
+                  const int* __restrict__ table, int table_stride, int ring_pages, T* __restrict__ pages, int chunk) {
   __shared__ float cs[DIFF_MAX_D / 2], sn[DIFF_MAX_D / 2];
   const int n = blockIdx.x;
   const int Q = 2 * H * d, K = 2 * G * d, V = G * dv;
   const int total = 2 * Q + K + V;
-  const int e0 = blockIdx.y * SPLIT_CHUNK;
-  const int e1 = min(total, e0 + SPLIT_CHUNK);
+  const int e0 = blockIdx.y * chunk;
+  const int e1 = min(total, e0 + chunk);
   const float* row = proj + (size_t)n * (Q + K + V);
   const int pos = row_pos[n];
   const int half = rot.rotary_dim / 2;
@@ -127,13 +127,16 @@ int tl_diff_split(const float* proj, const float* bias, const int* row_pos, cons
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "diff_split: unknown dtype code %d", dt);
   if (n == 0) return 0;
   const Rotation rot{inv_freq, rotary_dim, 0};
-  const dim3 grid(n, (4 * H * d + 2 * G * d + G * dv + SPLIT_CHUNK - 1) / SPLIT_CHUNK);
+  // few rows: chunks of SPLIT_CHUNK outputs, so that the row spreads over many workgroups; many rows: three workgroups a row
+  const int total = 4 * H * d + 2 * G * d + G * dv;
+  const int chunk = n >= 256 ? ((total + 2) / 3 + 255) / 256 * 256 : SPLIT_CHUNK;
+  const dim3 grid(n, (total + chunk - 1) / chunk);
   if (dt == DT_F32)
     diff_split_kernel<float><<<grid, 256, 0, st>>>(proj, bias, row_pos, rot, H, G, d, dv, (float*)q, (float*)k, (float*)v,
-                                                   table, table_stride, ring_pages, (float*)pages);
+                                                   table, table_stride, ring_pages, (float*)pages, chunk);
   else
     diff_split_kernel<bf16><<<grid, 256, 0, st>>>(proj, bias, row_pos, rot, H, G, d, dv, (bf16*)q, (bf16*)k, (bf16*)v,
-                                                  table, table_stride, ring_pages, (bf16*)pages);
+                                                  table, table_stride, ring_pages, (bf16*)pages, chunk);
   TL_LAUNCH_CHECK("diff_split");
   return 0;
 }

@@ -50,11 +50,11 @@ __global__ void __launch_bounds__(256)
 split_heads_kernel(const float* __restrict__ qf, int q_stride, const float* __restrict__ kf,
                    const float* __restrict__ vf, int kv_stride, const int* __restrict__ row_pos, int nq, int nkv,
                    int dk, int dv, T* __restrict__ q, T* __restrict__ k, T* __restrict__ v,
-                   const int* __restrict__ table, int table_stride, int ring_pages, T* __restrict__ pages) {
+                   const int* __restrict__ table, int table_stride, int ring_pages, T* __restrict__ pages, int chunk) {
   const int n = blockIdx.x;
   const int Q = nq * dk, K = nkv * dk, V = nkv * dv;
-  const int e0 = blockIdx.y * HEADS_CHUNK;
-  const int e1 = min(Q + K + V, e0 + HEADS_CHUNK);
+  const int e0 = blockIdx.y * chunk;
+  const int e1 = min(Q + K + V, e0 + chunk);
   T* kd = nullptr;
   T* vd = nullptr;
   int r = 0;
@@ -120,13 +120,16 @@ int tl_split_heads(const float* qf, int q_stride, const float* kf, const float* 
              "split_heads: pages without a page table");
   TL_REQUIRE(dt == DT_F32 || dt == DT_BF16, "split_heads: unknown dtype code %d", dt);
   if (n == 0) return 0;
-  const dim3 grid(n, (nq * dk + nkv * (dk + dv) + HEADS_CHUNK - 1) / HEADS_CHUNK);
+  // few rows: chunks of HEADS_CHUNK outputs, so that the row spreads over many workgroups; many rows: three workgroups a row
+  const int total = nq * dk + nkv * (dk + dv);
+  const int chunk = n >= 256 ? ((total + 2) / 3 + 255) / 256 * 256 : HEADS_CHUNK;
+  const dim3 grid(n, (total + chunk - 1) / chunk);
   if (dt == DT_F32)
     split_heads_kernel<float><<<grid, 256, 0, st>>>(qf, q_stride, kf, vf, kv_stride, row_pos, nq, nkv, dk, dv, (float*)q,
-                                                    (float*)k, (float*)v, table, table_stride, ring_pages, (float*)pages);
+                                                    (float*)k, (float*)v, table, table_stride, ring_pages, (float*)pages, chunk);
   else
     split_heads_kernel<bf16><<<grid, 256, 0, st>>>(qf, q_stride, kf, vf, kv_stride, row_pos, nq, nkv, dk, dv, (bf16*)q,
-                                                   (bf16*)k, (bf16*)v, table, table_stride, ring_pages, (bf16*)pages);
+                                                   (bf16*)k, (bf16*)v, table, table_stride, ring_pages, (bf16*)pages, chunk);
   TL_LAUNCH_CHECK("split_heads");
   return 0;
 }

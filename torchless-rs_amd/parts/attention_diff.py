@@ -72,6 +72,11 @@ class DifferentialAttentionMixer(Mixer):
     def may_capture(self, n_rows: int) -> bool:
         return self.proj is not None and self.proj.own_kernels(n_rows) and self.o.own_kernels(n_rows)
 
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        # few rows over a long context: the host cuts the keys into runs for workgroups of their own
+        return (self.proj is not None and self.dv == 2 * self.d and ops.prefill_serves(self.proj.weight.dtype, self.dv)
+                and ops.prefill_layout(n_new, len_before, self.window, 2 * self.nq, ops.compute_units(device)) is not None)
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         p, nm = self.prefix, self.names
         Q, K, V = 2 * self.nq * self.d, 2 * self.nkv * self.d, self.nkv * self.dv

@@ -221,19 +221,32 @@ def attend_and_commit(ctx, run, q: torch.Tensor, k, v, nkv: int, dk: int, dv: in
     and, unless every sequence brings one token (k and v are then None and lie in their pages
     already), this step's k [n, nkv, dk] and v [n, nkv, dv]: the step's rows attend to the pages
     for cached positions and to k and v for the new ones (values transposed by tiles where the
-    matrix cores run), and k and v are committed to the pages afterwards."""
+    matrix cores run), and k and v are committed to the pages afterwards.  Scores with no term but the
+    scale and the window go through the kernels of the attention without terms where the matrix cores
+    take the shape (one product with the values instead of two, and the keys of few rows over a long
+    context cut into runs)."""
     group = run.kv_group
     pages = group.storage[run.kv_layer]
     table = ctx.tables[run.kv_group_index]
+    cores = ops.scored_on_matrix_cores(ctx.dtype, dk, dv) and pages.dim() == 5
+    bare = cores and terms.slopes is None and terms.sinks is None and gate is None and att.dtype == ctx.dtype
     if ctx.all_single:
-        ops.attention_scored(q, None, None, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_after, terms, gate, att)
+        if bare:
+            ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after, terms.window, terms.scale, att)
+        else:
+            ops.attention_scored(q, None, None, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_after, terms, gate,
+                                 att)
         return
     vt = None
-    if ops.scored_on_matrix_cores(ctx.dtype, dk, dv):
+    if cores:
         vt = ctx.workspace.get("attend_vt" + tag, (nkv, dv, ctx.host["aligned_cols"]), ctx.dtype)
         ops.v_tiles_rows(v, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, ctx.len_after)
-    ops.attention_scored(q, k, v, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_before, terms, gate, att,
-                         vt_new=vt)
+    if bare:
+        ops.attention(q, k, v, pages, table, group.ring_pages, ctx, ctx.len_before, terms.window, terms.scale, att,
+                      vt_new=vt)
+    else:
+        ops.attention_scored(q, k, v, pages, nkv, dv, table, group.ring_pages, ctx, ctx.len_before, terms, gate, att,
+                             vt_new=vt)
     if vt is not None and pages.dim() == 5:       # values a tile at a time, in whole lines
         ops.kv_commit_tiles(k, vt, ctx.row_seq, ctx.row_pos, ctx.tile_off, ctx.len_before, ctx.len_after, table,
                             group.ring_pages, pages)

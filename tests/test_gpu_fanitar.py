@@ -51,8 +51,17 @@ ODD = {"architecture": "Fanitar", "vocab": 131, "width": 100, "norm": {"eps": 1e
            layer(diff(3, 3, 10, 12, 0.3, 0.4, rot=(300.0, 6), window=65), ff=36, limit=4.0),
            layer(diff(6, 2, 12, 20, 0.29, 0.2, rot=(20.0, 12))),
        ]}
-CONFIGS = {"mixed": MIXED, "cores": CORES, "ones": ONES, "odd": ODD}
-LENGTHS = {"mixed": [1, 7, 23, 70], "cores": [5, 64, 129, 330], "ones": [2, 65, 130, 200], "odd": [4, 33, 67, 140]}
+# head sizes that the matrix cores take but that are none of 64, 128 and 256 (48 and 80 wide, keys of two maps of
+# 24 and 40), three passes over the last two layers, a window of three pages and a bit
+HEADS = {"architecture": "Fanitar", "vocab": 300, "width": 192, "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
+         "logit_scale": 0.8, "loop": {"start": 1, "stop": 3, "times": 3}, "layers": [
+             layer(diff(6, 3, 24, 48, 0.2, 0.6, rot=(5000.0, 16)), ff=256, limit=2.0),
+             layer(latent(3, 48, 48, 72, 56, 0.15, window=200), ff=160, limit=1.0),
+             layer(diff(2, 1, 40, 80, 0.16, 0.45, rot=(100.0, 40)), ff=96, limit=6.0),
+         ]}
+CONFIGS = {"mixed": MIXED, "cores": CORES, "ones": ONES, "odd": ODD, "heads": HEADS}
+LENGTHS = {"mixed": [1, 7, 23, 70], "cores": [5, 64, 129, 330], "ones": [2, 65, 130, 200], "odd": [4, 33, 67, 140],
+           "heads": [3, 50, 131, 260]}
 NAMES = list(CONFIGS)
 
 
@@ -692,7 +701,7 @@ def test_unequal_batches_against_each_alone_with_slots_and_pages_used_again(zoo,
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["mixed", "ones", "cores"])
+@pytest.mark.parametrize("name", ["mixed", "ones", "cores", "heads"])
 def test_long_decoding_past_windows_and_rings(zoo, name, dtype):
     """A short prompt, then 300 tokens one by one (through captured graphs): every window is passed
     and every ring wraps more than once, in every pass's own cache."""

@@ -776,3 +776,117 @@ def test_the_command_line_and_the_trace_replay(zoo, tmp_path):
     want = z["want"][2]
     assert rel_err(first, torch.stack([want[0], want[19], want[2]])) < TOL["float32"]
     assert rel_err(last, want[21:22]) < TOL["float32"]
+
+
+# ---------------------------------------------------------------------------------------------
+# the new parts in a design of another arrangement
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_new_parts_serve_another_design(dtype):
+    """A model that is none of the designs, from the registry's parts alone, with old and new blocks
+    next to each other so that every kind of border between them is crossed: pre-norm around the older
+    attention with rotation and SwiGLU; the block with norms on both sides around the older attention
+    and SwiGLU, which do not know of it; pre-norm again; pre-norm around differential attention with a
+    subset of its options (no biases, no rotation, a window) and the clamped gate; norms on both sides
+    around attention out of latents without sink and gate and no feed-forward; the last two gone through
+    twice with the vector of a pass before each (and no embedding added again)."""
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.parts import LayerSpec, ModelSpec, PartSpec, Run
+    from torchless_rs_amd.weights import TensorDict, random_tensors
+    H, V, I, nq, nkv, d, eps, window = 64, 70, 96, 4, 2, 16, 1e-5, 20
+    rms = PartSpec("rmsnorm", {"size": H, "eps": eps})
+    rot = PartSpec("rotary", {"head_dim": d, "theta": 100.0})
+    swiglu = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I})
+    consts = {"alpha": 1.2, "limit": 1.5, "shift": 0.5}
+
+    def old_attention(position):
+        return PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d, "window": window,
+                                      "position": position})
+    pre = PartSpec("pre_norm", {"mixer_norm_name": "n1.", "ffn_norm_name": "n2."})
+    both = PartSpec("sandwich_norm", {"names": ("n1.", "n1b.", "n2.", "n2b.")})
+    layers = [
+        LayerSpec(prefix="h.0.", mixer=old_attention(rot), ffn=swiglu, mixer_norm=rms, ffn_norm=rms, block=pre),
+        LayerSpec(prefix="h.1.", mixer=old_attention(PartSpec("none", {})), ffn=swiglu, mixer_norm=rms, ffn_norm=rms,
+                  mixer_out_norm=rms, ffn_out_norm=rms, block=both),
+        LayerSpec(prefix="h.2.", mixer=old_attention(rot), ffn=swiglu, mixer_norm=rms, ffn_norm=rms, block=pre),
+        LayerSpec(prefix="h.3.", mixer=PartSpec("differential_attention", {
+            "hidden_size": H, "n_heads": 2, "n_kv_heads": 1, "head_dim": d, "v_head_dim": 2 * d, "lambda_init": 0.35,
+            "norm_eps": eps, "scale": 0.25, "window": 33}),
+            ffn=PartSpec("gated", {"hidden_size": H, "intermediate_size": I, "activation": "swish_clamped",
+                                   "activation_constants": consts}), mixer_norm=rms, ffn_norm=rms, block=pre),
+        LayerSpec(prefix="h.4.", mixer=PartSpec("latent_attention", {
+            "hidden_size": H, "n_heads": 2, "head_dim": d, "v_head_dim": 24, "q_rank": 20, "kv_rank": 12, "scale": 0.25,
+            "norm_eps": eps}), ffn=None, mixer_norm=rms, ffn_norm=None, mixer_out_norm=rms, block=both),
+    ]
+    schedule = [Run(0), Run(1), Run(2), Run(3, entry=(0, 0)), Run(4), Run(3, entry=(0, 1)), Run(4)]
+    spec = ModelSpec(hidden_size=H, vocab_size=V, embedding=PartSpec("tokens", {"vocab_size": V, "hidden_size": H, "scale": 2.0}),
+                     embedding_prefix="model.", layers=layers, schedule=schedule, final_norm=rms,
+                     final_norm_prefix="model.norm.", head=PartSpec("linear", {"vocab_size": V, "hidden_size": H}),
+                     head_prefix="lm_head.",
+                     stream_parts=[("passes.", PartSpec("pass_entry", {"hidden_size": H, "passes": 2, "name": "vec",
+                                                                       "add_embedding": False}))])
+    w = random_tensors(spec.weight_specs(), seed=6, std=0.2, norm_std=0.1, dtype=torch.bfloat16)
+    W = {k: v.double().cpu() for k, v in w.items()}
+    ids = some_prompts(V, [45], seed=9)[0]
+    n = len(ids)
+    pos = torch.arange(n)
+
+    def lin(name, t):
+        return t @ W[name].T
+
+    def older(p, y, rotated):
+        q, k, v = (lin(p + f"self_attn.{t}_proj.weight", y) for t in "qkv")
+        q, k = q.view(n, nq, d), k.view(n, nkv, d)
+        if rotated:
+            q, k = plain.rotate(q, pos, 100.0, d), plain.rotate(k, pos, 100.0, d)
+        k, v = k.repeat_interleave(nq // nkv, dim=1), v.view(n, nkv, d).repeat_interleave(nq // nkv, dim=1)
+        return lin(p + "self_attn.o_proj.weight", plain_heads(q, k, v, d ** -0.5, window).reshape(n, nq * d))
+
+    def silu_ffn(p, y):
+        g, u = lin(p + "mlp.gate_proj.weight", y), lin(p + "mlp.up_proj.weight", y)
+        return lin(p + "mlp.down_proj.weight", g / (1 + torch.exp(-g)) * u)
+
+    def norm(name, t):
+        return plain.rms(t, eps, W[name])
+
+    x = W["model.embed_tokens.weight"][ids] * 2.0
+    for p in ("h.0.", "h.1.", "h.2."):
+        if p == "h.1.":
+            x = x + norm(p + "n1b.weight", older(p, norm(p + "n1.weight", x), False))
+            x = x + norm(p + "n2b.weight", silu_ffn(p, norm(p + "n2.weight", x)))
+        else:
+            x = x + older(p, norm(p + "n1.weight", x), True)
+            x = x + silu_ffn(p, norm(p + "n2.weight", x))
+    zero = {"h.3.mix.q.b": torch.zeros(4 * d, dtype=torch.float64), "h.3.mix.k.b": torch.zeros(2 * d, dtype=torch.float64),
+            "h.3.mix.v.b": torch.zeros(2 * d, dtype=torch.float64), "h.4.mix.sink": torch.full((2,), -1e30, dtype=torch.float64),
+            "h.4.mix.g": torch.zeros(48, H, dtype=torch.float64)}
+    Wz = dict(W, **zero)
+    for t in range(2):
+        x = x + W["passes.vec"][t]
+        y = norm("h.3.n1.weight", x)
+        x = x + plain.differential_attention(y, Wz, "h.3.mix.", {"heads": 2, "kv_heads": 1, "dim": d, "vdim": 2 * d, "scale": 0.25,
+                                                                  "diff": 0.35, "mask": {"size": 33}}, eps)
+        y = norm("h.3.n2.weight", x)
+        g = lin("h.3.mlp.gate_proj.weight", y).clamp(max=1.5)
+        u = lin("h.3.mlp.up_proj.weight", y).clamp(-1.5, 1.5)
+        x = x + lin("h.3.mlp.down_proj.weight", g * torch.sigmoid(1.2 * g) * (u + 0.5))
+        y = norm("h.4.n1.weight", x)
+        # (no sink: one far below every score; no gate: a zero projection gates by one half, undone here)
+        a = plain.latent_attention(y, Wz, "h.4.mix.", {"heads": 2, "dim": d, "vdim": 24, "scale": 0.25}, eps) * 2.0
+        x = x + norm("h.4.n1b.weight", a)
+    want = lin("lm_head.weight", norm("model.norm.weight", x))
+    model = Model(spec, None, TORCH[dtype], torch.device("cuda:0"))
+    model.load_weights(TensorDict(w))
+    eng = Engine(model, max_tokens=256)
+    s = eng.alloc()
+    got = [eng.step([SeqInput(s, ids[:30], list(range(30)))]).clone()]
+    got += [eng.step([SeqInput(s, [t], [0])]).clone() for t in ids[30:]]       # (steps of one row: norms cut in two at the borders)
+    eng.free(s)
+    close(torch.cat(got), want, dtype, "old and new blocks side by side")
+    s = eng.alloc()
+    got = [eng.step([SeqInput(s, ids[at:at + 7], list(range(len(ids[at:at + 7]))))]).clone() for at in range(0, n, 7)]
+    eng.free(s)
+    close(torch.cat(got), want, dtype, "the same in portions of seven")
+    eng.close()

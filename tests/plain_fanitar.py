@@ -20,7 +20,7 @@ def rms(t, eps, w=None):
     return y if w is None else y * w
 
 
-def visible(T, window=None, first_row=0):
+def visible(T, window=None):
     """[T, T] bool: row p sees column j iff j <= p and (with a window) p - j < window."""
     p = torch.arange(T)[:, None]
     j = torch.arange(T)[None, :]

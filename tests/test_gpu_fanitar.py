@@ -304,8 +304,8 @@ class Sequence:
         self.ws = Workspace(torch.device("cuda"))
         self.length = 0
 
-    def step(self, n_new, make):
-        """`make(ctx, pages_or_none, table, ring)` -> (q, k, v): the mixer's split for this step's rows."""
+    def step(self, n_new):
+        """(ctx, run) of a step that brings `n_new` rows after what the sequence holds."""
         from torchless_rs_amd.kernels import ops
         i32 = dict(dtype=torch.int32, device="cuda")
         cached = self.length
@@ -331,7 +331,7 @@ def latent_steps(dtype, H, dk, dv, window, sinks, q, k, v, cuts, scale=1.0):
     terms = ops.ScoreTerms(scale, window, None, dev(sinks.float()) if sinks is not None else None)
     outs, at = [], 0
     for n in cuts:
-        ctx, run = seq.step(n, None)
+        ctx, run = seq.step(n)
         qf = dev(q[at:at + n].reshape(n, H * dk).float())
         kvf = dev(torch.cat([k[at:at + n].reshape(n, -1), v[at:at + n].reshape(n, -1)], dim=1).float())
         qs = torch.empty(n, H, dk, dtype=seq.dt, device="cuda")
@@ -423,7 +423,7 @@ def diff_steps(dtype, H, G, d, dv, window, lam, post, eps, proj, cuts, scale=1.0
     terms = ops.ScoreTerms(scale, window, None, None)
     outs, at = [], 0
     for n in cuts:
-        ctx, run = seq.step(n, None)
+        ctx, run = seq.step(n)
         pr = dev(proj[at:at + n].float().contiguous())
         qs = torch.empty(n, 2 * H, 2 * d, dtype=seq.dt, device="cuda")
         maps = torch.empty(n, 2 * H, dv, dtype=seq.dt, device="cuda")

@@ -76,11 +76,12 @@ class PassEntry(StreamPart):
 
     def load(self, tensors, compute_dtype) -> None:
         self.table = tensors[self.name].to(torch.float32).contiguous()
+        self.rows = [self.table[t] for t in range(self.passes)]
 
     def forward(self, ctx, x: torch.Tensor, embedded, t: int) -> None:
         if not (0 <= t < self.passes):
             raise ValueError(f"pass {t} of {self.passes}")
-        ops.stream_entry(x, embedded if (t > 0 and self.needs_embedding) else None, self.table[t])
+        ops.stream_entry(x, embedded if (t > 0 and self.needs_embedding) else None, self.rows[t])
 
 
 register_part("stream", "pass_entry", PassEntry)
